@@ -59,10 +59,13 @@ class ScheduleEntry:
     that another layer's run owns; None means the layer's own.  `cache_id` gives this run a
     cache and state of its own under that number, whatever layer's weights it runs with (a
     layer that is run again with the same tensors, as a layer of its own: ids and the indices
-    of layers that own a cache share one numbering, so an id is no such layer's index)."""
+    of layers that own a cache share one numbering, so an id is no such layer's index).  `before`: a stream op
+    (a `PartSpec` of that registry) that runs on the residual stream right before this run, e.g. what a pass over a
+    span of layers adds to the stream when it starts."""
     layer: int
     cache_of: Optional[int] = None
     cache_id: Optional[int] = None
+    before: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)

@@ -8,7 +8,9 @@
 //
 // Options of the score, each off unless given:  s = (q . k) * scale;  with a soft cap c,
 // s = c * tanh(s / c);  with per-head slopes a[h], s -= a[h] * (p - p') (a bias that grows
-// with the distance to the key).
+// with the distance to the key).  With per-head `sinks` z[h] the softmax's denominator also holds
+// exp(z[h]): one more weight, taken as it is, that no value goes with.  With `values_in_keys`
+// there is no V pool: a key's first dv dims are its value (attention over a latent).
 //
 // Reference: PagedAttention::forward at /root/reference/src/models/layers/attention.rs:947-958
 // (external kernel); golden formula tests/probes/compare_flashinfer_probe.py:51-73:
@@ -22,17 +24,19 @@
 
 namespace xi {
 
-constexpr int kMaxHeadDim = 256;
+constexpr int kMaxHeadDim = 256;       // heads up to this size take the first instantiation,
+constexpr int kMaxHeadDimWide = 640;   // up to this the second
 constexpr int kAttnWaves = 4;
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, T* __restrict__ out, float scale, int window, int page_size,
-    int nq, int nkv, int d, int dv, int v_grouped, float softcap, const float* __restrict__ slopes) {
-  __shared__ float q_s[kMaxHeadDim];
-  __shared__ float acc_s[kAttnWaves][kMaxHeadDim];
+    int nq, int nkv, int d, int dv, int v_grouped, float softcap, const float* __restrict__ slopes,
+    const float* __restrict__ sinks, int values_in_keys) {
+  __shared__ float q_s[MAXD];
+  __shared__ float acc_s[kAttnWaves][MAXD];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
 
   const int t = blockIdx.x;
@@ -51,7 +55,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
   const float slope = slopes ? slopes[h] : 0.f;
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
 
-  constexpr int NE = kMaxHeadDim / kWave;  // output dims per lane
+  constexpr int NE = MAXD / kWave;  // output dims per lane
   float acc[NE];
 #pragma unroll
   for (int e = 0; e < NE; ++e) acc[e] = 0.f;
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
       const int rj = __shfl(row, j, kWave);
       const int vrj = __shfl(vrow, j, kWave);
       const int voj = __shfl(voff, j, kWave);
-      const T* vp = v_cache + (size_t)rj * dv;
+      const T* vp = values_in_keys ? k_cache + (size_t)rj * d : v_cache + (size_t)rj * dv;
       const T* vtp = v_cache + (size_t)vrj * page_size + (size_t)(voj >> 3) * dv * 8 + (voj & 7);  // [offset / 8, dv, 8] block
 #pragma unroll
       for (int e = 0; e < NE; ++e) {
@@ -115,6 +119,8 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
   float mm = m_s[0];
 #pragma unroll
   for (int w = 1; w < kAttnWaves; ++w) mm = fmaxf(mm, m_s[w]);
+  const float sink = sinks ? sinks[h] : -INFINITY;
+  mm = fmaxf(mm, sink);
   float f[kAttnWaves];
   float ll = 0.f;
 #pragma unroll
@@ -122,6 +128,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     f[w] = (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm);
     ll += l_s[w] * f[w];
   }
+  if (sinks) ll += expf(sink - mm);
   T* op = out + ((size_t)t * nq + h) * dv;
   for (int i = threadIdx.x; i < dv; i += blockDim.x) {
     float o = 0.f;
@@ -140,27 +147,29 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
                                     const int* tok_seq, const int* positions, void* out,
                                     float scale, int window, int page_size, int n_tok, int nq,
                                     int nkv, int d, int dv, int v_grouped, float softcap, const float* slopes,
-                                    hipStream_t stream) {
+                                    const float* sinks, int values_in_keys, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && page_size > 0 && max_pages > 0,
            "attention: bad sizes T=%d nq=%d nkv=%d page=%d max_pages=%d", n_tok, nq, nkv, page_size, max_pages);
   XI_CHECK(nq % nkv == 0, "attention: %d query heads are not a multiple of %d kv heads", nq, nkv);
-  XI_CHECK(d > 0 && d <= kMaxHeadDim, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDim);
-  XI_CHECK(dv > 0 && dv <= kMaxHeadDim, "attention: value head size %d is outside 1..%d", dv, kMaxHeadDim);
+  XI_CHECK(d > 0 && d <= kMaxHeadDimWide, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDimWide);
+  XI_CHECK(dv > 0 && dv <= kMaxHeadDimWide, "attention: value head size %d is outside 1..%d", dv, kMaxHeadDimWide);
+  XI_CHECK(!values_in_keys || (dv <= d && !v_grouped), "attention: values that are the keys' first dims need dv <= d");
   XI_CHECK(softcap >= 0.f, "attention: the soft cap must be positive (0: none), got %g", (double)softcap);
   XI_CHECK(nq <= 65535, "attention: too many heads (%d)", nq);
   XI_CHECK(!v_grouped || page_size % 8 == 0, "attention: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d", page_size);
   if (n_tok == 0) return 0;
   dim3 grid(n_tok, nq);
-  if (dtype == kF32)
-    attention_generic_kernel<float><<<grid, kAttnWaves * kWave, 0, stream>>>(
-        (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (float*)out, scale, window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes);
-  else if (dtype == kBF16)
-    attention_generic_kernel<bf16><<<grid, kAttnWaves * kWave, 0, stream>>>(
-        (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (bf16*)out, scale, window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes);
-  else
-    XI_CHECK(false, "attention: unknown dtype %d", dtype);
+  const bool wide = d > kMaxHeadDim || dv > kMaxHeadDim;
+#define XI_AG(TT, MAXD)                                                                                                 \
+  attention_generic_kernel<TT, MAXD><<<grid, kAttnWaves * kWave, 0, stream>>>(                                          \
+      (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, block_tables, max_pages, tok_seq, positions, (TT*)out, scale, \
+      window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes, sinks, values_in_keys)
+  if (dtype == kF32 && !wide) XI_AG(float, kMaxHeadDim);
+  else if (dtype == kF32) XI_AG(float, kMaxHeadDimWide);
+  else if (dtype == kBF16 && !wide) XI_AG(bf16, kMaxHeadDim);
+  else if (dtype == kBF16) XI_AG(bf16, kMaxHeadDimWide);
+  else XI_CHECK(false, "attention: unknown dtype %d", dtype);
+#undef XI_AG
   XI_LAUNCH_CHECK("attention_generic");
   return 0;
 }

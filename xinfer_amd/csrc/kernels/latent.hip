@@ -1,0 +1,191 @@
+// Attention over a latent: what a token keeps is one vector c (rank dims, the RMS-normed first part of a down
+// projection) and one rotated key part (r dims) shared by all heads; a head's keys and values are products of c
+// with matrices of its own, U_k [dim, rank] and U_v [vdim, rank].  Both products move to the query's side:
+//
+//   score(i, j) = ((U_k^T q_plain_i) . c_j + q_turned_i . k_turned_j) * scale        o_i = U_v (sum_j p_ij c_j)
+//
+// so the attention itself is one kv head with keys [c | k_turned] of rank + r dims whose first `rank` dims are
+// the values too, read from one pool [pages, 1, page, rank + r].
+//
+// `latent_rows_kernel`, a workgroup a token, from the packed projection row [q (H (dim + r)) | down (rank + r) | ..]:
+//   c = down[:rank] / sqrt(mean(down[:rank]^2) + eps) * w   and the turned down[rank:] into the pool at the slot;
+//   every head's turned q part into q_full[t, h, rank:].
+// Pairs (2i, 2i + 1) or (i, i + r / 2) turn by the position's row of float32 tables [positions, r / 2].
+//
+// `head_linear_kernel`: out[t, h, n] = sum_k x[t, h, k] * w[h][n][k] for every head, with the strides of all
+// three given (U_k is read as [k][n], U_v as [n][k]); float32 sums in ascending k (a tile of 32 at a time); with a
+// gate, out *= sigmoid(gate[t, h, n]).
+#include "common.h"
+
+namespace xi {
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ proj, long long proj_stride, int q_off,
+                                                          int down_off, const float* __restrict__ w, float eps,
+                                                          const long long* __restrict__ slots, T* __restrict__ pool,
+                                                          int page_size, T* __restrict__ q_full, int H, int dim, int r,
+                                                          int rank, const float* __restrict__ cos_t,
+                                                          const float* __restrict__ sin_t, int interleaved,
+                                                          const int* __restrict__ positions) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * proj_stride;
+  const int half = r / 2;
+  const size_t trow = (size_t)positions[t] * half;
+  // the heads' turned parts
+  T* qf = q_full + (size_t)t * H * (rank + r);
+  for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
+    const int h = i / half, p = i - h * half;
+    const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
+    const T* src = row + q_off + (size_t)h * (dim + r) + dim;
+    const float a = to_float(src[ia]), b = to_float(src[ib]);
+    const float cs = cos_t[trow + p], sn = sin_t[trow + p];
+    T* dst = qf + (size_t)h * (rank + r) + rank;
+    dst[ia] = from_float<T>(a * cs - b * sn);
+    dst[ib] = from_float<T>(b * cs + a * sn);
+  }
+  const T* down = row + down_off;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float v = to_float(down[i]);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = rsqrtf(block_sum<4>(ss, scratch) / (float)rank + eps);
+  const long long slot = slots[t];
+  if (slot < 0) return;
+  T* dst = pool + (size_t)slot * (rank + r);       // [pages, 1, page, rank + r]: slot = page * page_size + offset
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) dst[i] = from_float<T>(to_float(down[i]) * inv * w[i]);
+  for (int p = threadIdx.x; p < half; p += blockDim.x) {
+    const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
+    const float a = to_float(down[rank + ia]), b = to_float(down[rank + ib]);
+    const float cs = cos_t[trow + p], sn = sin_t[trow + p];
+    dst[rank + ia] = from_float<T>(a * cs - b * sn);
+    dst[rank + ib] = from_float<T>(b * cs + a * sn);
+  }
+}
+
+constexpr int kHlRows = 32, kHlCols = 64, kHlK = 32;
+
+// a workgroup of 256 threads: 32 tokens by 64 outputs of one head; a thread 2 tokens by 4 outputs
+template <typename T>
+__global__ __launch_bounds__(256) void head_linear_kernel(const T* __restrict__ x, long long x_row, long long x_head,
+                                                          const T* __restrict__ w, long long w_head, long long w_n,
+                                                          long long w_k, T* __restrict__ out, long long o_row,
+                                                          long long o_head, const T* __restrict__ gate, long long g_row,
+                                                          long long g_head, int n_tok, int N, int K) {
+  __shared__ float xs[kHlK][kHlRows + 1];
+  __shared__ float ws[kHlK][kHlCols + 1];
+  const int h = blockIdx.z;
+  const int t0 = blockIdx.x * kHlRows, n0 = blockIdx.y * kHlCols;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;       // outputs n0 + tx + 16 j, tokens t0 + ty + 16 i
+  float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  const T* xh = x + (size_t)h * x_head;
+  const T* wh = w + (size_t)h * w_head;
+  for (int k0 = 0; k0 < K; k0 += kHlK) {
+    for (int e = threadIdx.x; e < kHlK * kHlRows; e += 256) {
+      const int tt = e / kHlK, kk = e - tt * kHlK;              // k fastest: x's k is contiguous
+      const int t = t0 + tt, k = k0 + kk;
+      xs[kk][tt] = (t < n_tok && k < K) ? to_float(xh[(size_t)t * x_row + k]) : 0.f;
+    }
+    for (int e = threadIdx.x; e < kHlK * kHlCols; e += 256) {
+      int nn, kk;
+      if (w_k == 1) {                                           // k contiguous
+        nn = e / kHlK;
+        kk = e - nn * kHlK;
+      } else {                                                  // n contiguous
+        kk = e / kHlCols;
+        nn = e - kk * kHlCols;
+      }
+      const int n = n0 + nn, k = k0 + kk;
+      ws[kk][nn] = (n < N && k < K) ? to_float(wh[(size_t)n * w_n + (size_t)k * w_k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < kHlK; ++kk) {
+      const float a0 = xs[kk][ty], a1 = xs[kk][ty + 16];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float b = ws[kk][tx + 16 * j];
+        acc[0][j] = fmaf(a0, b, acc[0][j]);
+        acc[1][j] = fmaf(a1, b, acc[1][j]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int t = t0 + ty + 16 * i;
+    if (t >= n_tok) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (gate) {
+        const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + n]);
+        v *= 1.f / (1.f + expf(-g));
+      }
+      out[(size_t)t * o_row + (size_t)h * o_head + n] = from_float<T>(v);
+    }
+  }
+}
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+// proj rows of proj_stride elements: the heads' q parts [H, dim + r] from q_off, the down projection [rank + r] from
+// down_off; w float32 [rank]; pool [pages, 1, page, rank + r]; q_full [T, H, rank + r] (its last r dims are written).
+int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_off, int dtype, const float* w, float eps,
+                   const long long* slots, void* pool, int page_size, void* q_full, int n_tok, int H, int dim, int r, int rank,
+                   const float* cos_t, const float* sin_t, int interleaved, const int* positions, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && dim > 0 && r >= 0 && r % 2 == 0 && rank > 0 && page_size > 0,
+           "latent_rows: bad sizes T=%d H=%d dim=%d r=%d rank=%d page=%d", n_tok, H, dim, r, rank, page_size);
+  XI_CHECK(q_off >= 0 && down_off >= 0 && proj_stride >= (long long)q_off + (long long)H * (dim + r) &&
+               proj_stride >= (long long)down_off + rank + r,
+           "latent_rows: the projection's rows are too short");
+  XI_CHECK(r == 0 || (cos_t && sin_t), "latent_rows: a rotation needs its tables");
+  XI_CHECK(w && positions && slots, "latent_rows: the norm's weight, the positions and the slots are needed");
+  if (n_tok == 0) return 0;
+  if (dtype == kF32)
+    latent_rows_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)proj, proj_stride, q_off, down_off, w, eps, slots,
+                                                         (float*)pool, page_size, (float*)q_full, H, dim, r, rank, cos_t,
+                                                         sin_t, interleaved, positions);
+  else if (dtype == kBF16)
+    latent_rows_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)proj, proj_stride, q_off, down_off, w, eps, slots,
+                                                        (bf16*)pool, page_size, (bf16*)q_full, H, dim, r, rank, cos_t, sin_t,
+                                                        interleaved, positions);
+  else
+    XI_CHECK(false, "latent_rows: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("latent_rows");
+  return 0;
+}
+
+// x: token t, head h, element k at x + t x_row + h x_head + k; w: head h, output n, element k at w + h w_head + n w_n +
+// k w_k (one of w_n, w_k is 1); out: at out + t o_row + h o_head + n; gate null or laid out like out with its own strides.
+int xi_head_linear(const void* x, long long x_row, long long x_head, const void* w, long long w_head, long long w_n,
+                   long long w_k, void* out, long long o_row, long long o_head, const void* gate, long long g_row,
+                   long long g_head, int dtype, int n_tok, int H, int N, int K, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0 && N > 0 && K > 0, "head_linear: bad sizes T=%d H=%d N=%d K=%d", n_tok, H, N, K);
+  XI_CHECK(w_n == 1 || w_k == 1, "head_linear: the weight's outputs or its inputs must lie side by side");
+  XI_CHECK(H <= 65535, "head_linear: too many heads");
+  if (n_tok == 0) return 0;
+  dim3 grid((unsigned)((n_tok + kHlRows - 1) / kHlRows), (unsigned)((N + kHlCols - 1) / kHlCols), (unsigned)H);
+  XI_CHECK(grid.y <= 65535u, "head_linear: too many outputs");
+  if (dtype == kF32)
+    head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)w, w_head, w_n, w_k,
+                                                        (float*)out, o_row, o_head, (const float*)gate, g_row, g_head, n_tok,
+                                                        N, K);
+  else if (dtype == kBF16)
+    head_linear_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)x, x_row, x_head, (const bf16*)w, w_head, w_n, w_k,
+                                                       (bf16*)out, o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N,
+                                                       K);
+  else
+    XI_CHECK(false, "head_linear: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("head_linear");
+  return 0;
+}
+
+}  // extern "C"

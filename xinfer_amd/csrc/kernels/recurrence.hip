@@ -7,7 +7,12 @@
 //   per head   a_t[i] = decay[h] for every token and channel (retention),
 //   per token  a_t[i] = sigmoid(z_t[h, i])^(1 / tau) = exp(-softplus(-z) / tau), z float32 [T, H dk]
 //              plus a bias [H dk] (gated linear attention); the logarithm, the exponential and the state
+//              are float32;
+//   per token and head   a_t[i] = exp(-exp(A[h]) * d_t) for every channel, with the step size d_t = softplus(raw_t[h] +
+//              bias[h]) (no clamp) from a column of the projection; the value row is multiplied by d_t as it is read
+//              (a selective state space: S <- a_t S + d_t k_t v_t^T).  Step size, exponentials and the product d_t v_t
 //              are float32.
+// With `group_heads` g > 1, q and k have one set of dk columns for every g heads (head h reads set h / g).
 // q, k and v are columns of a packed projection (a row stride and a column offset each); q and k are
 // multiplied by `q_scale` / `k_scale` in float32 as they are read.
 //
@@ -48,7 +53,8 @@ template <typename T, int RPT>
 __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
     long long v_stride, const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau,
-    const float* __restrict__ head_decay,
+    const float* __restrict__ head_decay, const T* __restrict__ step, long long step_stride,
+    const float* __restrict__ step_bias, const float* __restrict__ decay_log, int group_heads,
     const float* __restrict__ state_in, long long in_stride, const long long* __restrict__ in_idx,
     float* __restrict__ state_out, long long out_stride, const long long* __restrict__ out_idx,
     const int* __restrict__ first, const int* __restrict__ last, float* __restrict__ out, float* __restrict__ decay_out,
@@ -72,17 +78,26 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   const int c = threadIdx.x;            // the channel this thread fetches for the workgroup
   const float hd = head_decay ? head_decay[h] : 0.f;
   const float zb = (z_bias && c < dk) ? z_bias[h * dk + c] : 0.f;
-  auto fetch = [&](int t, float& fq, float& fk, float& fa) {      // (channels past the head's stay zero)
+  const int qk0 = (h / group_heads) * dk;       // the head's set of q and k columns
+  const float sb = step ? step_bias[h] : 0.f, rate = step ? -expf(decay_log[h]) : 0.f;
+  // the token's step size (1 where the decay has another source): every thread makes its own copy
+  auto step_of = [&](int t) {
+    if (!step) return 1.f;
+    const float x = to_float(step[(size_t)t * step_stride + h]) + sb;
+    return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
+  };
+  auto fetch = [&](int t, float dt, float& fq, float& fk, float& fa) {      // (channels past the head's stay zero)
     if (c < dk) {
-      fq = to_float(q[(size_t)t * q_stride + h * dk + c]) * q_scale;
-      fk = to_float(k[(size_t)t * k_stride + h * dk + c]) * k_scale;
-      fa = z ? decay_of(z[((size_t)t * H + h) * dk + c] + zb, inv_tau) : hd;
+      fq = to_float(q[(size_t)t * q_stride + qk0 + c]) * q_scale;
+      fk = to_float(k[(size_t)t * k_stride + qk0 + c]) * k_scale;
+      fa = step ? expf(rate * dt) : z ? decay_of(z[((size_t)t * H + h) * dk + c] + zb, inv_tau) : hd;
     }
   };
   float fq = 0.f, fk = 0.f, fa = 0.f;
-  fetch(t0, fq, fk, fa);
+  float dt = step_of(t0);
+  fetch(t0, dt, fq, fk, fa);
   // the token's value is asked for a token ahead as well: no step of the walk waits for memory
-  float v_next = col ? to_float(v[(size_t)t0 * v_stride + h * dv + j]) : 0.f;
+  float v_next = col ? to_float(v[(size_t)t0 * v_stride + h * dv + j]) * dt : 0.f;
   qs[0][c] = fq;
   ks[0][c] = fk;
   as[0][c] = fa;
@@ -92,8 +107,9 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     all_decays *= fa;
     const float vj = v_next;
     if (t + 1 < t1) {
-      fetch(t + 1, fq, fk, fa);
-      if (col) v_next = to_float(v[(size_t)(t + 1) * v_stride + h * dv + j]);
+      dt = step_of(t + 1);
+      fetch(t + 1, dt, fq, fk, fa);
+      if (col) v_next = to_float(v[(size_t)(t + 1) * v_stride + h * dv + j]) * dt;
     }
     float acc = 0.f;
     const float4* a4 = reinterpret_cast<const float4*>(&as[cur][wave * RPT]);
@@ -183,20 +199,27 @@ using namespace xi;
 
 extern "C" {
 
-// q, k [T, .] with H dk columns from the given pointers, v with H dv, rows `*_stride` elements apart, in `dtype`;
-// z float32 [T, H dk] (z_bias float32 [H dk] or null) or null (then head_decay float32 [H]).  Item w walks tokens
+// q, k [T, .] with H dk columns from the given pointers (H / group_heads sets of dk columns if group_heads > 1), v with
+// H dv, rows `*_stride` elements apart, in `dtype`; the decay from z float32 [T, H dk] (z_bias float32 [H dk] or null), or
+// from head_decay float32 [H], or from step (rows of step_stride elements in `dtype`, H columns: the raw step sizes) with
+// step_bias and decay_log float32 [H]: one of the three.  Item w walks tokens
 // first[w] .. last[w] - 1 from the state state_in + in_idx[w] * in_stride ([H, dk, dv] float32; in_idx null or a
 // negative entry: from zeros) and leaves its last state at state_out + out_idx[w] * out_stride (null or negative:
 // nowhere); out float32 [T, H, dv] or null (no results); decay_out float32 [items, H, dk] or null: the product of
 // each channel's decays over the item.
 int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v, long long v_stride,
-                   int dtype, const float* z, const float* z_bias, float tau, const float* head_decay, const float* state_in,
+                   int dtype, const float* z, const float* z_bias, float tau, const float* head_decay, const void* step,
+                   long long step_stride, const float* step_bias, const float* decay_log, int group_heads,
+                   const float* state_in,
                    long long in_stride, const long long* in_idx, float* state_out, long long out_stride,
                    const long long* out_idx, const int* first, const int* last, float* out, float* decay_out, int n_items, int H,
                    int dk, int dv, float q_scale, float k_scale, hipStream_t stream) {
   XI_CHECK(n_items >= 0 && H > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes items=%d H=%d dk=%d dv=%d", n_items, H, dk, dv);
   XI_CHECK(dk <= kScanWaves * 64, "linear_scan: key heads of up to %d channels, not %d", kScanWaves * 64, dk);
-  XI_CHECK((z != nullptr) != (head_decay != nullptr), "linear_scan: a decay per token or a decay per head, one of them");
+  XI_CHECK((z != nullptr) + (head_decay != nullptr) + (step != nullptr) == 1,
+           "linear_scan: a decay per token and channel, per head, or per token and head from a step size: one of them");
+  XI_CHECK(step == nullptr || (step_bias && decay_log && step_stride >= H), "linear_scan: a step size needs its bias and its rate");
+  XI_CHECK(group_heads >= 1 && H % group_heads == 0, "linear_scan: %d heads in groups of %d", H, group_heads);
   XI_CHECK(z == nullptr || tau > 0.f, "linear_scan: tau must be positive");
   XI_CHECK((in_idx == nullptr || (state_in && in_stride >= (long long)H * dk * dv)) &&
                (out_idx == nullptr || (state_out && out_stride >= (long long)H * dk * dv)),
@@ -209,7 +232,8 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
   const int rpt = (dk + kScanWaves - 1) / kScanWaves;
 #define XI_SCAN(TT, R)                                                                                                        \
   linear_scan_kernel<TT, R><<<grid, kScanWaves * kWave, 0, stream>>>(                                                         \
-      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, state_in, in_stride, \
+      (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, (const TT*)step,    \
+      step_stride, step_bias, decay_log, group_heads, state_in, in_stride,                                                    \
       in_idx, state_out, out_stride, out_idx, first, last, out, decay_out, H, dk, dv, q_scale, k_scale)
 #define XI_SCAN_T(TT)            \
   do {                           \

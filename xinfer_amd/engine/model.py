@@ -16,7 +16,9 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..parts import (KVNeed, LayerCache, StateNeed, StepContext, Stream, block_class, embedding_class,
-                     head_class, norm_class)
+                     head_class, norm_class, state_needs_of, stream_op_class)
+
+EMBEDDING_CACHE = -1        # the key of the state that the embedding keeps (no layer's index, no run's cache id)
 from ..weights.store import TensorDecl, WeightStore
 
 
@@ -37,6 +39,12 @@ class CausalLM:
         self.blocks = [block_class(l.block)(l, dtype) for l in spec.layers]
         self.final_norm = norm_class(spec.final_norm.kind)(spec.final_norm, dtype)
         self.head = head_class(spec.head.kind)(spec.head, dtype)
+        # what runs on the stream before a schedule entry's layer: one object a distinct spec
+        self.stream_ops = {}
+        for e in spec.schedule:
+            if e.before is not None and id(e.before) not in self.stream_ops:
+                self.stream_ops[id(e.before)] = stream_op_class(e.before.kind)(e.before, dtype)
+        self._keep_first = any(op.needs_first for op in self.stream_ops.values())
         for e in spec.schedule:
             if not (0 <= e.layer < len(self.blocks)):
                 raise ValueError(f"schedule names layer {e.layer} but the model has {len(self.blocks)}")
@@ -51,7 +59,7 @@ class CausalLM:
     @property
     def graph_safe(self) -> bool:
         """Every part can be recorded into a HIP graph (see `Part.graph_safe`)."""
-        return all(p.graph_safe for p in (self.embedding, self.final_norm, self.head, *self.blocks))
+        return all(p.graph_safe for p in (self.embedding, self.final_norm, self.head, *self.blocks, *self.stream_ops.values()))
 
     # ---- weights -------------------------------------------------------------
     @classmethod
@@ -59,6 +67,9 @@ class CausalLM:
         decls = embedding_class(spec.embedding.kind).declare(spec.embedding)
         for l in spec.layers:
             decls += block_class(l.block).declare(l)
+        for e in spec.schedule:
+            if e.before is not None:
+                decls += stream_op_class(e.before.kind).declare(e.before, "")
         decls += norm_class(spec.final_norm.kind).declare(spec.final_norm, str(spec.final_norm.get("prefix", "")))
         decls += head_class(spec.head.kind).declare(spec.head)
         seen, out = set(), []
@@ -79,6 +90,8 @@ class CausalLM:
         self.embedding.load(store, "", device)
         for b in self.blocks:
             b.load(store, device)
+        for op in self.stream_ops.values():
+            op.load(store, "", device)
         self.final_norm.load(store, str(self.spec.final_norm.get("prefix", "")), device)
         self.head.load(store, "", device, shared=self.embedding.table if self.head.tied else None)
         return self
@@ -88,7 +101,7 @@ class CausalLM:
         """Which runs own pages, in which group; which own per-request state.  A cache is known by a key:
         the layer's index, or the `cache_id` of a run that keeps one of its own."""
         self.kv_needs: Dict[int, KVNeed] = {}
-        self.state_needs: Dict[int, StateNeed] = {}
+        self.state_needs: Dict[int, StateNeed] = {}      # a cache's state, or a tuple of them if its part keeps several
         layer_of: Dict[int, int] = {}
         for e in self.spec.schedule:
             if e.cache_of is None:
@@ -115,6 +128,8 @@ class CausalLM:
             st = self.blocks[l].state_need()
             if st is not None:
                 self.state_needs[key] = st
+        if state_needs_of(self.embedding.state_need()):
+            self.state_needs[EMBEDDING_CACHE] = self.embedding.state_need()
         self.cache_groups: List[CacheGroupNeed] = [
             CacheGroupNeed(w, tuple(by_window[w])) for w in windows]
         self.group_of_layer: Dict[int, int] = {
@@ -132,7 +147,11 @@ class CausalLM:
                 want_rows: torch.Tensor) -> torch.Tensor:
         """ids int32 [T]; caches: layer index -> the cache that layer owns; want_rows int32
         [R].  Returns float32 logits [R, vocab]."""
-        first = self.embedding.forward(ids, ctx)
+        if EMBEDDING_CACHE in self.state_needs:
+            first = self.embedding.forward(ids, ctx, cache=caches[EMBEDDING_CACHE])
+        else:
+            first = self.embedding.forward(ids, ctx)
+        kept_first = first.clone() if self._keep_first else None       # the norms add into `first` in place
         # an embedding kind may also hand on its result rounded to the activation dtype (`rows`)
         stream = Stream(first, None, rows=getattr(self.embedding, "rows", None))
         schedule = self.spec.schedule
@@ -141,12 +160,16 @@ class CausalLM:
             if c is None:
                 c = LayerCache()
             elif e.cache_of is not None:
-                c = LayerCache(c.group, c.pools, c.state, write=False)
+                c = LayerCache(c.group, c.pools, c.state, write=False, states=c.states)
+            if e.before is not None:
+                stream = self.stream_ops[id(e.before)].forward(stream, kept_first, ctx)
             blk = self.blocks[e.layer]
             if getattr(blk, "folds", False):
                 # the block that runs next may let this one half do its first norm
                 nxt = self.blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
                 next_norm = nxt.first_norm() if getattr(nxt, "folds", False) else None
+                if nxt is not None and schedule[i + 1].before is not None:
+                    next_norm = None          # something changes the stream in between: the norm sees another sum
                 stream = blk.forward(stream, ctx, c, next_norm=next_norm)
             else:
                 stream = blk.forward(stream, ctx, c)

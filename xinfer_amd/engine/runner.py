@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from ..cache import DecodeStepError, BatchArrays, CacheGroup, PagedCacheManager
-from ..parts import LayerCache, StepContext
+from ..parts import LayerCache, StepContext, state_needs_of
 from .model import CausalLM
 
 
@@ -184,13 +184,14 @@ class ModelRunner:
                 pools[pool.name] = torch.zeros(shape, dtype=pool.dtype or model.dtype, device=self.device)
             self.layer_caches[layer] = LayerCache(group=g, pools=pools)
         self._state_arenas: List[torch.Tensor] = []
-        for layer, st in model.state_needs.items():
-            arena = torch.zeros((self.max_requests, *st.shape), dtype=st.dtype, device=self.device)
-            self._state_arenas.append(arena)
-            if layer in self.layer_caches:
-                self.layer_caches[layer].state = arena
-            else:
-                self.layer_caches[layer] = LayerCache(state=arena)
+        for layer, need in model.state_needs.items():
+            for st in state_needs_of(need):      # one arena a named state; the first is the cache's `state`
+                arena = torch.zeros((self.max_requests, *st.shape), dtype=st.dtype, device=self.device)
+                self._state_arenas.append(arena)
+                c = self.layer_caches.setdefault(layer, LayerCache())
+                if c.state is None:
+                    c.state = arena
+                c.states[st.name] = arena
         self._empty_f32 = torch.empty((1, 0), dtype=torch.float32, device=self.device)
         self._staging = _Staging(self.device)
         self.use_graphs = bool(use_graphs) and model.graph_safe

@@ -277,10 +277,12 @@ def scan_chunk_plan(q_lens, chunk: Optional[int] = None):
     return whole, long, chunks
 
 
-def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, state_in, in_stride, in_idx, state_out, out_stride, out_idx,
+def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, group_heads,
+                 state_in, in_stride, in_idx, state_out, out_stride, out_idx,
                  first, last, out, decay_out, items, H, dk, dv, q_scale, k_scale):
     _ok(lib().xi_linear_scan(_p(q), ctypes.c_longlong(qs), _p(k), ctypes.c_longlong(ks), _p(v), ctypes.c_longlong(vs),
-                             _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay), _p(state_in),
+                             _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay),
+                             _p(step), ctypes.c_longlong(ss), _p(step_bias), _p(decay_log), int(group_heads), _p(state_in),
                              ctypes.c_longlong(in_stride), _p(in_idx), _p(state_out), ctypes.c_longlong(out_stride),
                              _p(out_idx), ctypes.c_void_p(first), ctypes.c_void_p(last), _p(out), _p(decay_out), int(items),
                              H, dk, dv, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _stream()))
@@ -289,11 +291,16 @@ def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, state_in, in_s
 def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
                 cu_q: torch.Tensor, heads: int, key_dim: int, value_dim: int, z: Optional[torch.Tensor] = None,
                 tau: float = 1.0, head_decay: Optional[torch.Tensor] = None, q_scale: float = 1.0,
-                k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None, q_lens=None, plan_cache=None) -> torch.Tensor:
+                k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None, q_lens=None, plan_cache=None,
+                step: Optional[torch.Tensor] = None, step_bias: Optional[torch.Tensor] = None,
+                decay_log: Optional[torch.Tensor] = None, groups: Optional[int] = None) -> torch.Tensor:
     """Linear attention with a decaying float32 state per request and head, S <- diag(a) S + k v^T, o = S^T q,
     token by token from the state each request's slot holds (left there afterwards).  q, k [T, H dk] and
     v [T, H dv] may be column ranges of a packed projection.  The decay: `z` float32 [T, H dk], `z_bias`
-    float32 [H dk] (or None) and `tau` (a = sigmoid(z + bias)^(1 / tau) per token and key channel) or `head_decay` float32 [H] (a constant per head).
+    float32 [H dk] (or None) and `tau` (a = sigmoid(z + bias)^(1 / tau) per token and key channel) or `head_decay` float32 [H] (a constant per head),
+    or `step` [T, H] (columns of a projection, in q's type), `step_bias` and `decay_log` float32 [H]: the step size d =
+    softplus(step + step_bias), a = exp(-exp(decay_log) d) per token and head, and the token's value row times d.
+    `groups` G: q and k are [T, G dk] and head h reads the columns of group h // (H / G).
     state float32 [slots, H, dk, dv] (slots may be strided); state_slots int64 [B]; cu_q int32 [B + 1].
     Returns o float32 [T, H, dv].
     `q_lens` (the host's copy of the portions' lengths; None: nothing of the step is read on the host, as a step
@@ -303,15 +310,31 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     the index arrays of this cutting are kept for the next layer."""
     H, dk, dv = int(heads), int(key_dim), int(value_dim)
     T = q.shape[0]
-    qs, ks, vs = _columns(q, H * dk, "linear_scan: q"), _columns(k, H * dk, "linear_scan: k"), _columns(v, H * dv, "linear_scan: v")
+    G = H if groups is None else int(groups)
+    if G <= 0 or H % G:
+        raise KernelError(f"linear_scan: {H} heads in {G} groups")
+    qs, ks, vs = _columns(q, G * dk, "linear_scan: q"), _columns(k, G * dk, "linear_scan: k"), _columns(v, H * dv, "linear_scan: v")
     if k.shape[0] != T or v.shape[0] != T or q.dtype != k.dtype or q.dtype != v.dtype or not (q.device == k.device == v.device):
         raise KernelError("linear_scan: q, k and v must be rows of the same tokens, type and device")
-    _dev(z, head_decay, state_slots, cu_q, z_bias)
+    _dev(z, head_decay, state_slots, cu_q, z_bias, step_bias, decay_log)
+    ss = 0
+    if step is not None:
+        if z is not None or head_decay is not None or step_bias is None or decay_log is None:
+            raise KernelError("linear_scan: a step size comes with its bias and its rate, and alone")
+        ss = _columns(step, H, "linear_scan: step")
+        if step.shape[0] != T or step.dtype != q.dtype or step.device != q.device:
+            raise KernelError("linear_scan: the step sizes must be rows of the same tokens, type and device")
+        for t_, what in ((step_bias, "step_bias"), (decay_log, "decay_log")):
+            _want(t_, torch.float32, f"linear_scan: {what}")
+            if t_.shape != (H,):
+                raise KernelError(f"linear_scan: {what} {tuple(t_.shape)} must be [{H}]")
     if z_bias is not None and (z is None or z_bias.dtype != torch.float32 or z_bias.shape != (H * dk,)):
         raise KernelError(f"linear_scan: the bias of the decay's logits must be float32 [{H * dk}], beside z")
-    if (z is None) == (head_decay is None):
+    if step is None and (z is None) == (head_decay is None):
         raise KernelError("linear_scan: a decay per token (z) or per head (head_decay), one of them")
-    if z is not None:
+    if step is not None:
+        pass
+    elif z is not None:
         _want(z, torch.float32, "linear_scan: z")
         if z.shape != (T, H * dk) or not tau > 0:
             raise KernelError(f"linear_scan: z {tuple(z.shape)} must be [{T}, {H * dk}] and tau positive")
@@ -332,7 +355,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
         raise KernelError("linear_scan: the portions' lengths do not add up to the step's tokens")
     out = torch.empty((T, H, dv), dtype=torch.float32, device=q.device)
     slot_stride = int(state.stride(0)) if state.shape[0] > 1 else H * dk * dv
-    common = (q, k, v, qs, ks, vs, z, z_bias, tau, head_decay)
+    common = (q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, H // G)
     whole, long, chunks = scan_chunk_plan(q_lens) if q_lens is not None else (None, [], [])
     if not long:            # every request in one piece, straight from the step's own arrays
         _scan_launch(*common, state, slot_stride, state_slots, state, slot_stride, state_slots, cu_q.data_ptr(),
@@ -739,23 +762,35 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
                       scale: float, window: int = 0, out: Optional[torch.Tensor] = None,
                       v_grouped: bool = False, softcap: float = 0.0,
-                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      slopes: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
+                      value_dim: Optional[int] = None) -> torch.Tensor:
     """Causal paged GQA attention for any mix of tokens.  q [T, nq, d]; caches
     [pages, nkv, page_size, d] (the V pool's last size, the value head size, may differ);
     block_tables int32 [B, max_pages]; tok_seq / positions
     int32 [T] name each token's row of block_tables and its absolute position.
     window = 0 keeps all keys, w > 0 the last w (the query's own key included).
     `softcap` c > 0: scores become c * tanh(score / c); `slopes` float32 [nq]: head h's scores lose
-    slopes[h] * (distance from the query to the key)."""
-    _dev(q, k_cache, v_cache, block_tables, tok_seq, positions, out, slopes)
+    slopes[h] * (distance from the query to the key); `sinks` float32 [nq]: head h's softmax has exp(sinks[h]) in
+    its denominator beside the keys' weights.  `v_cache` None: a key's first `value_dim` dims are its value (one
+    pool for both: attention over a latent)."""
+    _dev(q, k_cache, v_cache, block_tables, tok_seq, positions, out, slopes, sinks)
     if q.dim() != 3:
         raise KernelError("attention: q must be [T, nq, d]")
     T, nq, d = q.shape
     if k_cache.dim() != 4:
         raise KernelError("attention: the K pool must be [pages, nkv, page_size, d]")
     nkv, page = k_cache.shape[1], k_cache.shape[2]
-    dv = int(v_cache.shape[3])
-    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention", dv=dv)
+    if v_cache is None:
+        dv = int(value_dim or 0)
+        if not (0 < dv <= d) or v_grouped or k_cache.shape[3] != d or k_cache.dtype != q.dtype:
+            raise KernelError(f"attention: values inside the keys need 0 < value_dim <= {d} and a pool [pages, nkv, page, {d}]")
+    else:
+        dv = int(v_cache.shape[3])
+        _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention", dv=dv)
+    if sinks is not None:
+        _want(sinks, torch.float32, "attention: sinks")
+        if sinks.shape != (nq,):
+            raise KernelError(f"attention: sinks {tuple(sinks.shape)} must be one a query head, [{nq}]")
     for t, name in ((block_tables, "block_tables"), (tok_seq, "tok_seq"), (positions, "positions")):
         _want(t, torch.int32, f"attention: {name}")
     if block_tables.dim() != 2 or tok_seq.shape != (T,) or positions.shape != (T,):
@@ -773,7 +808,8 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _ok(lib().xi_attention_generic(
         _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
         int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
-        int(window), int(page), T, nq, nkv, d, dv, int(bool(v_grouped)), ctypes.c_float(softcap), _p(slopes), _stream()))
+        int(window), int(page), T, nq, nkv, d, dv, int(bool(v_grouped)), ctypes.c_float(softcap), _p(slopes), _p(sinks),
+        int(v_cache is None), _stream()))
     return out
 
 
@@ -1582,3 +1618,225 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if out_dtype == torch.float32:
         return torch.mm(x, w.t(), out_dtype=torch.float32)
     return torch.nn.functional.linear(x, w)
+
+
+# ---- an embedding that looks at the token before; what a run of layers adds when it starts ----------------
+def embed_pair(table: torch.Tensor, pairs: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+               cu_q: torch.Tensor, state_slots: torch.Tensor, last: torch.Tensor, scale: float, buckets: int,
+               mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """out[t] = float32(table[ids[t]]) * scale + float32(pairs[row(t)]), row(t) = (prev * mul_prev + ids[t] * mul_cur)
+    mod buckets with prev the token before t in its sequence, and row `buckets` at position 0.  The token before a
+    portion's first token is `last[state_slots[b]]` (int32 [slots]: what `keep_last_token` left there)."""
+    _dev(table, pairs, ids, positions, tok_seq, cu_q, state_slots, last)
+    for t, name in ((ids, "ids"), (positions, "positions"), (tok_seq, "tok_seq"), (cu_q, "cu_q"), (last, "last")):
+        _want(t, torch.int32, f"embed_pair: {name}")
+    _want(state_slots, torch.int64, "embed_pair: state_slots")
+    if table.dim() != 2 or pairs.dim() != 2 or pairs.shape[1] != table.shape[1] or pairs.dtype != table.dtype:
+        raise KernelError("embed_pair: table [V, H] and pairs [buckets + 1, H] of one type")
+    T, H, B = ids.shape[0], table.shape[1], state_slots.shape[0]
+    if int(buckets) <= 0 or pairs.shape[0] != int(buckets) + 1 or int(mul_prev) < 0 or int(mul_cur) < 0:
+        raise KernelError(f"embed_pair: {pairs.shape[0]} rows of pairs for {buckets} buckets and one more")
+    if positions.shape != (T,) or tok_seq.shape != (T,) or cu_q.shape != (B + 1,) or last.dim() != 1:
+        raise KernelError("embed_pair: positions and tok_seq [T], cu_q [B + 1], last [slots]")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _ok(lib().xi_embed_pair(_p(table), _p(pairs), _code(table, "embed_pair"), _p(ids), _p(positions), _p(tok_seq), _p(cu_q),
+                            _p(state_slots), _p(last), _p(out), T, H, ctypes.c_float(scale), ctypes.c_longlong(int(buckets)),
+                            ctypes.c_longlong(int(mul_prev)), ctypes.c_longlong(int(mul_cur)), _stream()))
+    return out
+
+
+def keep_last_token(ids: torch.Tensor, cu_q: torch.Tensor, state_slots: torch.Tensor, last: torch.Tensor) -> None:
+    """last[state_slots[b]] = the last token of sequence b's portion in this step."""
+    _dev(ids, cu_q, state_slots, last)
+    for t, name in ((ids, "ids"), (cu_q, "cu_q"), (last, "last")):
+        _want(t, torch.int32, f"keep_last_token: {name}")
+    _want(state_slots, torch.int64, "keep_last_token: state_slots")
+    B = state_slots.shape[0]
+    if cu_q.shape != (B + 1,) or last.dim() != 1 or ids.dim() != 1:
+        raise KernelError("keep_last_token: ids [T], cu_q [B + 1], last [slots]")
+    _ok(lib().xi_keep_last_token(_p(ids), _p(cu_q), _p(state_slots), _p(last), B, _stream()))
+
+
+def stream_start(resid: torch.Tensor, pending: Optional[torch.Tensor], factor: float, first: Optional[torch.Tensor],
+                 vec: Optional[torch.Tensor]) -> torch.Tensor:
+    """resid += factor * pending (+ first) (+ vec), in place, float32: `pending` rows [T, H] in either precision or a
+    stack [P, T, H] of float32 partial sums (or None), `first` float32 [T, H] or None, `vec` float32 [H] or None."""
+    _dev(resid, pending, first, vec)
+    _want(resid, torch.float32, "stream_start: the stream")
+    if resid.dim() != 2:
+        raise KernelError("stream_start: the stream must be [T, H]")
+    T, H = resid.shape
+    parts, code = 1, F32
+    if pending is not None:
+        if pending.dim() == 3:
+            _want(pending, torch.float32, "stream_start: partial sums")
+            parts = int(pending.shape[0])
+        if tuple(pending.shape[-2:]) != (T, H) or pending.dim() not in (2, 3):
+            raise KernelError(f"stream_start: the branch {tuple(pending.shape)} does not fit the stream {(T, H)}")
+        code = _code(pending, "stream_start")
+    if first is not None and (first.dtype != torch.float32 or tuple(first.shape) != (T, H)):
+        raise KernelError("stream_start: the embedding's output must be float32 [T, H]")
+    if vec is not None and (vec.dtype != torch.float32 or tuple(vec.shape) != (H,)):
+        raise KernelError("stream_start: the vector must be float32 [H]")
+    _ok(lib().xi_stream_start(_p(resid), _p(pending), code, parts, ctypes.c_float(factor), _p(first), _p(vec), T, H, _stream()))
+    return resid
+
+
+# ---- a projection's heads made ready one by one: rotation, then a unit norm ---------------------------------
+def head_rows(qkv: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, num_heads: int,
+              num_kv_heads: int, head_dim: int, value_dim: int, v_grouped: bool = False, cos: Optional[torch.Tensor] = None,
+              sin: Optional[torch.Tensor] = None, rotary_dim: int = 0, interleaved: bool = False,
+              positions: Optional[torch.Tensor] = None, unit_norm: bool = False, eps: float = 0.0) -> torch.Tensor:
+    """A packed projection [T, nq d + nkv d + nkv dv]: the first `rotary_dim` dims of every q and k head turn by the
+    token's position (pairs (2i, 2i + 1) if `interleaved`, else (i, i + r / 2); `cos` / `sin` float32 [positions, r / 2]),
+    then, with `unit_norm`, each head is divided by its root mean square over d (eps inside the root); k and v go into
+    the paged cache at `slots`.  Returns q [T, nq, d]."""
+    _dev(qkv, slots, k_cache, v_cache, cos, sin, positions)
+    nq, nkv, d, dv, rot = int(num_heads), int(num_kv_heads), int(head_dim), int(value_dim), int(rotary_dim)
+    if qkv.dim() != 2 or qkv.shape[1] != nq * d + nkv * d + nkv * dv:
+        raise KernelError(f"head_rows: qkv {tuple(qkv.shape)} is not [T, {nq * d + nkv * d + nkv * dv}]")
+    T = qkv.shape[0]
+    _want(slots, torch.int64, "head_rows: slots")
+    if slots.shape != (T,) or d > 1024:
+        raise KernelError("head_rows: slots must be [T]; heads of up to 1024 dims")
+    if rot:
+        if rot % 2 or not (0 < rot <= d) or cos is None or sin is None or positions is None:
+            raise KernelError(f"head_rows: {rot} rotated dims of a head of {d} need tables and positions")
+        _want(cos, torch.float32, "head_rows: cos")
+        _want(sin, torch.float32, "head_rows: sin")
+        _want(positions, torch.int32, "head_rows: positions")
+        if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != rot // 2 or positions.shape != (T,):
+            raise KernelError(f"head_rows: the rotation's tables must be [positions, {rot // 2}], positions [T]")
+    _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_grouped, "head_rows", dv=dv)
+    q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
+    _ok(lib().xi_head_rows(_p(qkv), _code(qkv, "head_rows"), _p(slots), _p(q_out), _p(k_cache), _p(v_cache),
+                           int(k_cache.shape[2]), T, nq, nkv, d, dv, int(bool(v_grouped)), _p(cos if rot else None),
+                           _p(sin if rot else None), rot, int(bool(interleaved)), _p(positions if rot else None),
+                           int(bool(unit_norm)), ctypes.c_float(eps), _stream()))
+    return q_out
+
+
+# ---- attention over a latent ---------------------------------------------------------------------------------
+def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight: torch.Tensor, eps: float,
+                slots: torch.Tensor, pool: torch.Tensor, q_full: torch.Tensor, heads: int, dim: int, rot_dim: int,
+                rank: int, cos: torch.Tensor, sin: torch.Tensor, interleaved: bool, positions: torch.Tensor) -> None:
+    """From the packed projection `proj` [T, W] (the heads' q parts [H, dim + rot_dim] from column `q_offset`, the down
+    projection [rank + rot_dim] from `down_offset`): the latent = RMSNorm(down[:rank]) * norm_weight and the turned
+    down[rank:] into `pool` [pages, 1, page, rank + rot_dim] at `slots`; every head's turned q part into
+    q_full[:, h, rank:] (q_full [T, H, rank + rot_dim])."""
+    _dev(proj, norm_weight, slots, pool, q_full, cos, sin, positions)
+    H, d, r, rank = int(heads), int(dim), int(rot_dim), int(rank)
+    if proj.dim() != 2 or q_full.dtype != proj.dtype or pool.dtype != proj.dtype:
+        raise KernelError("latent_rows: the projection, the pool and q of one type")
+    T, W = proj.shape
+    if q_offset < 0 or down_offset < 0 or q_offset + H * (d + r) > W or down_offset + rank + r > W:
+        raise KernelError(f"latent_rows: rows of {W} do not hold the q parts and the down projection")
+    if tuple(q_full.shape) != (T, H, rank + r) or pool.dim() != 4 or pool.shape[1] != 1 or pool.shape[3] != rank + r:
+        raise KernelError(f"latent_rows: q {tuple(q_full.shape)} must be [{T}, {H}, {rank + r}], the pool [pages, 1, page, {rank + r}]")
+    _want(norm_weight, torch.float32, "latent_rows: the norm's weight")
+    _want(slots, torch.int64, "latent_rows: slots")
+    _want(positions, torch.int32, "latent_rows: positions")
+    _want(cos, torch.float32, "latent_rows: cos")
+    _want(sin, torch.float32, "latent_rows: sin")
+    if (norm_weight.shape != (rank,) or slots.shape != (T,) or positions.shape != (T,) or r % 2 or cos.shape != sin.shape
+            or cos.dim() != 2 or cos.shape[1] != r // 2):
+        raise KernelError(f"latent_rows: weight [{rank}], slots and positions [T], tables [positions, {r // 2}]")
+    _ok(lib().xi_latent_rows(_p(proj), ctypes.c_longlong(W), int(q_offset), int(down_offset), _code(proj, "latent_rows"),
+                             _p(norm_weight), ctypes.c_float(eps), _p(slots), _p(pool), int(pool.shape[2]), _p(q_full), T, H,
+                             d, r, rank, _p(cos), _p(sin), int(bool(interleaved)), _p(positions), _stream()))
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, h, n] = sum_k x[t, h, k] * w[h, n, k] for every head, float32 sums in ascending k; with `gate`
+    [T, H, N], out *= sigmoid(gate).  All operands may be strided views ([T, H, .] of packed rows; w [H, N, K] with
+    either N or K contiguous) of one type; `out` [T, H, N] is written in place."""
+    for t in (x, w, out, gate):
+        if t is not None and (not t.is_cuda or t.dtype != x.dtype or t.device != x.device):
+            raise KernelError("head_linear: operands of one type on one GPU")
+    if x.dim() != 3 or w.dim() != 3 or out.dim() != 3:
+        raise KernelError("head_linear: x [T, H, K], w [H, N, K], out [T, H, N]")
+    T, H, K = x.shape
+    N = w.shape[1]
+    if tuple(w.shape) != (H, N, K) or tuple(out.shape) != (T, H, N) or (gate is not None and tuple(gate.shape) != (T, H, N)):
+        raise KernelError(f"head_linear: x {tuple(x.shape)}, w {tuple(w.shape)} and out {tuple(out.shape)} do not match")
+    if x.stride(2) != 1 or out.stride(2) != 1 or (gate is not None and gate.stride(2) != 1) or 1 not in (w.stride(1), w.stride(2)):
+        raise KernelError("head_linear: the last axis of x, out and the gate, and N or K of w, must be contiguous")
+    ll = ctypes.c_longlong
+    g = gate if gate is not None else out
+    _ok(lib().xi_head_linear(_p(x), ll(x.stride(0)), ll(x.stride(1)), _p(w), ll(w.stride(0)), ll(w.stride(1)), ll(w.stride(2)),
+                             _p(out), ll(out.stride(0)), ll(out.stride(1)), _p(gate), ll(g.stride(0)), ll(g.stride(1)),
+                             _code(x, "head_linear"), T, H, N, K, _stream()))
+    return out
+
+
+# ---- around the state of a selective state-space mixer ---------------------------------------------------------
+def causal_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, tails: torch.Tensor, state_slots: torch.Tensor,
+                tok_seq: torch.Tensor, cu_q: torch.Tensor) -> torch.Tensor:
+    """out[t, c] = silu(bias[c] + sum_j weight[c, j] u[t - (taps - 1) + j, c]) within each sequence; inputs from before
+    the step's portion come from the request's tail (`tails` float32 [slots, taps - 1, C], oldest first; slots may be
+    strided), which is left as it is (`conv_tail` moves it on).  u [T, C] may be columns of a packed projection;
+    weight float32 [C, taps], bias float32 [C].  Returns [T, C] in u's type."""
+    _dev(weight, bias, state_slots, tok_seq, cu_q)
+    T, C = u.shape
+    us = _columns(u, C, "causal_conv: u")
+    _want(weight, torch.float32, "causal_conv: weight")
+    _want(bias, torch.float32, "causal_conv: bias")
+    _want(tails, torch.float32, "causal_conv: tails")
+    _want(state_slots, torch.int64, "causal_conv: state_slots")
+    _want(tok_seq, torch.int32, "causal_conv: tok_seq")
+    _want(cu_q, torch.int32, "causal_conv: cu_q")
+    taps = int(weight.shape[1]) if weight.dim() == 2 else 0
+    B = state_slots.shape[0]
+    if weight.dim() != 2 or weight.shape[0] != C or taps < 1 or bias.shape != (C,) or tok_seq.shape != (T,) or cu_q.shape != (B + 1,):
+        raise KernelError(f"causal_conv: weight [{C}, taps], bias [{C}], tok_seq [T], cu_q [B + 1]")
+    if (tails.dim() != 3 or tuple(tails.shape[1:]) != (taps - 1, C) or not tails.is_cuda or tails.device != u.device
+            or (taps > 1 and tails[0].stride() != (C, 1))):
+        raise KernelError(f"causal_conv: tails {tuple(tails.shape)} must be [slots, {taps - 1}, {C}] with whole slots")
+    out = torch.empty((T, C), dtype=u.dtype, device=u.device)
+    stride = int(tails.stride(0)) if tails.shape[0] > 1 else (taps - 1) * C
+    _ok(lib().xi_causal_conv(_p(u), ctypes.c_longlong(us), _code(u, "causal_conv"), _p(weight), _p(bias), _p(tails),
+                             ctypes.c_longlong(stride), _p(state_slots), _p(tok_seq), _p(cu_q), _p(out), T, C, taps, _stream()))
+    return out
+
+
+def conv_tail(u: torch.Tensor, tails: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor) -> None:
+    """Moves every request's tail on by its portion of this step: afterwards it holds the last taps - 1 inputs."""
+    _dev(state_slots, cu_q)
+    T, C = u.shape
+    us = _columns(u, C, "conv_tail: u")
+    _want(tails, torch.float32, "conv_tail: tails")
+    _want(state_slots, torch.int64, "conv_tail: state_slots")
+    _want(cu_q, torch.int32, "conv_tail: cu_q")
+    B = state_slots.shape[0]
+    if tails.dim() != 3 or tails.shape[2] != C or cu_q.shape != (B + 1,) or not tails.is_cuda or tails.device != u.device:
+        raise KernelError(f"conv_tail: tails {tuple(tails.shape)} must be [slots, taps - 1, {C}], cu_q [B + 1]")
+    taps = int(tails.shape[1]) + 1
+    if taps > 1 and tails[0].stride() != (C, 1):
+        raise KernelError("conv_tail: whole slots")
+    stride = int(tails.stride(0)) if tails.shape[0] > 1 else (taps - 1) * C
+    _ok(lib().xi_conv_tail(_p(u), ctypes.c_longlong(us), _code(u, "conv_tail"), _p(tails), ctypes.c_longlong(stride),
+                           _p(state_slots), _p(cu_q), B, C, taps, _stream()))
+
+
+def gated_group_norm(y: torch.Tensor, x: torch.Tensor, skip: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float,
+                     groups: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """v = (y + skip[h] x) * silu(z), then each of `groups` equal parts of a row divided by its root mean square (eps
+    inside the root), times `weight`.  y float32 [T, H, dv]; x, z [T, H dv] in `out_dtype` (may be columns of packed
+    rows); skip float32 [H]; weight float32 [H dv].  Returns [T, H dv] in `out_dtype`."""
+    _dev(y, skip, weight)
+    _want(y, torch.float32, "gated_group_norm: y")
+    if y.dim() != 3:
+        raise KernelError("gated_group_norm: y must be [T, H, dv]")
+    T, H, dv = y.shape
+    W = H * dv
+    xs, zs = _columns(x, W, "gated_group_norm: x"), _columns(z, W, "gated_group_norm: z")
+    if x.shape[0] != T or z.shape[0] != T or x.dtype != out_dtype or z.dtype != out_dtype or x.device != y.device or z.device != y.device:
+        raise KernelError("gated_group_norm: x and z must be rows of the same tokens in the output's type")
+    _want(skip, torch.float32, "gated_group_norm: skip")
+    _want(weight, torch.float32, "gated_group_norm: weight")
+    if skip.shape != (H,) or weight.shape != (W,) or int(groups) <= 0 or W % int(groups):
+        raise KernelError(f"gated_group_norm: skip [{H}], weight [{W}], and groups that divide {W}")
+    out = torch.empty((T, W), dtype=out_dtype, device=y.device)
+    _ok(lib().xi_gated_group_norm(_p(y), _p(x), ctypes.c_longlong(xs), _p(skip), _p(z), ctypes.c_longlong(zs), _p(weight),
+                                  ctypes.c_float(eps), _p(out), _code(out, "gated_group_norm"), T, W, dv, int(groups), _stream()))
+    return out

@@ -18,6 +18,12 @@ scalar tensor of the layer); other tensor names (`names`).  Any of these takes t
 the attention kernels that know the score's options follow.  That kernel also rotates q and k by
 position (pairs (i, i + rotary_dim / 2), float32 tables) where the spec names a position encoding and
 no q/k norm.
+
+`qk_norm="head_unit"`: every q and k head is divided by its root mean square over head_dim (`qk_norm_eps` inside the
+root), without a weight, AFTER the rotation.  A rotation turns pairs of dims and leaves a head's sum of squares as it
+is, so the plain form computes this with its own kernels (norm with a weight of ones, then rotation: the same but for
+rounding); with the options of the paragraph above, or with `general=True`, a kernel that takes a head at a time does
+it in the order given (`kernels.head_rows`: rotation of either pairing, then the unit norm, then the cache write).
 """
 from __future__ import annotations
 
@@ -51,6 +57,7 @@ class PagedAttention(Mixer):
         self.scale = float(spec.get("scale", self.d ** -0.5))
         self.dv = int(spec.get("value_dim") or self.d)
         self.row_norm = spec.get("qk_norm") == "row"
+        self.unit_norm = spec.get("qk_norm") == "head_unit"
         self.softcap = float(spec.get("score_softcap") or 0.0)
         slopes = spec.get("distance_slopes")
         self.slope_values = None if slopes is None else tuple(float(a) for a in slopes)
@@ -63,13 +70,20 @@ class PagedAttention(Mixer):
         self.slopes = None           # float32 [nq] on the device
         # the options that the fused q/k kernel and the attention kernels of the plain form do not know
         self.general = bool(self.dv != self.d or self.row_norm or self.softcap > 0 or self.slope_values is not None
-                            or self.value_mix_key is not None)
-        if self.general and spec.get("position") is not None and (self.qk_norm or bool(spec["position"].get("interleaved", False))):
+                            or self.value_mix_key is not None or spec.get("general", False))
+        interleaved = spec.get("position") is not None and bool(spec["position"].get("interleaved", False))
+        # the general form's heads are made ready a head at a time where they are normed one by one or turned in pairs
+        # (2i, 2i + 1); else a row at a time
+        self.by_head = self.general and (self.unit_norm or interleaved)
+        if self.by_head and (self.row_norm or self.value_mix_key is not None):
+            raise NotImplementedError("attention whose heads are normed one by one or turned in pairs (2i, 2i + 1) takes no "
+                                      "norm over the whole projection and no blended values")
+        if self.general and not self.by_head and spec.get("position") is not None and self.qk_norm:
             raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size takes a "
                                       "rotation of the pairs (i, i + rotary_dim / 2) and then no q/k norm")
-        if self.general and (self.qk_norm and not self.row_norm or self.bias):
+        if self.general and (self.qk_norm and not (self.row_norm or self.unit_norm) or self.bias):
             raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size "
-                                      "takes the q/k norm over the whole projection or none, and no biases")
+                                      "takes the q/k norm over the whole projection, the heads' unit norm or none, and no biases")
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
         # A step of single tokens reads nothing on the host where the split-K decode kernel or the
@@ -109,7 +123,7 @@ class PagedAttention(Mixer):
                     TensorDecl(n["v_bias"], (nkv * dv,))]
         if spec.get("qk_norm") == "row":
             out += [TensorDecl(n["q_norm"], (nq * d,), "norm"), TensorDecl(n["k_norm"], (nkv * d,), "norm")]
-        elif spec.get("qk_norm", False):
+        elif spec.get("qk_norm", False) and spec.get("qk_norm") != "head_unit":
             out += [TensorDecl(n["q_norm"], (d,), "norm"), TensorDecl(n["k_norm"], (d,), "norm")]
         vm = spec.get("value_mix")
         if vm and not vm.get("source", False):
@@ -128,7 +142,9 @@ class PagedAttention(Mixer):
         if self.bias:
             self.qkv_bias = torch.cat([store.get(names[f"{n}_bias"], torch.float32, device)
                                        for n in ("q", "k", "v")]).contiguous()
-        if self.qk_norm:
+        if self.unit_norm:         # the plain form's kernels norm with a weight: ones
+            self.q_norm_w = self.k_norm_w = None if self.general else torch.ones(self.d, dtype=torch.float32, device=device)
+        elif self.qk_norm:
             self.q_norm_w = store.get(names["q_norm"], torch.float32, device).contiguous()
             self.k_norm_w = store.get(names["k_norm"], torch.float32, device).contiguous()
         if self.value_mix_key is not None and not self.value_mix_source:
@@ -201,6 +217,15 @@ class PagedAttention(Mixer):
                 if v_other is None:
                     raise RuntimeError(f"values {self.value_mix_key!r} are blended in before the layer that makes them has run")
         pos = self.position
+        if self.by_head:
+            q = kernels.head_rows(qkv, slots, cache.k, cache.v, self.nq, self.nkv, self.d, self.dv, v_grouped=vt,
+                                  cos=pos.cos if pos is not None else None, sin=pos.sin if pos is not None else None,
+                                  rotary_dim=pos.rotary_dim if pos is not None else 0,
+                                  interleaved=pos.interleaved if pos is not None else False, positions=ctx.positions,
+                                  unit_norm=self.unit_norm, eps=self.qk_norm_eps)
+            a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt,
+                                  softcap=self.softcap, slopes=self.slopes)
+            return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)
         q = kernels.qkv_rows(qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps, slots, cache.k, cache.v,
                              self.nq, self.nkv, self.d, self.dv, v_grouped=vt, v_other=v_other, mix=self.mix,
                              cos=pos.cos if pos is not None else None, sin=pos.sin if pos is not None else None,

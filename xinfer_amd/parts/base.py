@@ -25,6 +25,8 @@ runs on the tokens of one step.  A part never learns which model it is in.
                    ignores it); `table` is what a tied head shares
   Head             forward(h) -> float32 logits [R, vocab]; load(..., shared=) takes the
                    embedding's table when the spec says `tied`
+  StreamOp         forward(stream, first, ctx) -> stream: a change of the stream between two runs
+                   of layers (what a pass over a span of layers adds when it starts)
 
 New kinds register themselves with the decorators below; a `PartSpec.kind` then selects
 them.  Nothing else in the engine has to change.
@@ -87,9 +89,22 @@ class KVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Fixed-size state per live request: one slot of this shape and dtype."""
+    """Fixed-size state per live request: one slot of this shape and dtype.  A part that keeps several (a
+    matrix and the last inputs of a convolution, say) returns a tuple of them from `state_need`, each with a
+    `name` of its own; the first is `LayerCache.state`, all are in `LayerCache.states` by name."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    name: str = "state"
+
+
+def state_needs_of(need) -> Tuple["StateNeed", ...]:
+    """What `state_need()` returned (None, one StateNeed, or several) as a tuple with names of their own."""
+    if need is None:
+        return ()
+    needs = (need,) if isinstance(need, StateNeed) else tuple(need)
+    if len({n.name for n in needs}) != len(needs):
+        raise ValueError("the states of one part need names of their own")
+    return needs
 
 
 @dataclass
@@ -98,8 +113,9 @@ class LayerCache:
     the cache that another layer's run owns."""
     group: int = -1
     pools: Dict[str, torch.Tensor] = field(default_factory=dict)   # by PoolNeed.name: [pages, *shape]
-    state: Optional[torch.Tensor] = None      # [max_requests, *StateNeed.shape]
+    state: Optional[torch.Tensor] = None      # [max_requests, *StateNeed.shape] (the first, if the part keeps several)
     write: bool = True
+    states: Dict[str, torch.Tensor] = field(default_factory=dict)   # by StateNeed.name
 
     @property
     def k(self) -> Optional[torch.Tensor]:
@@ -239,7 +255,22 @@ class PositionEncoding(Part):
 class TokenEmbedding(Part):
     table: Optional[torch.Tensor] = None
 
+    def state_need(self) -> Optional[StateNeed]:
+        """Fixed-size state per live request that the embedding itself keeps (the token before, say); a kind that
+        returns one gets `forward(ids, ctx, cache=LayerCache)` with its slots."""
+        return None
+
     def forward(self, ids: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class StreamOp(Part):
+    """Something that changes the residual stream between two runs of layers (`ScheduleEntry.before`):
+    forward(stream, first, ctx) -> stream, with `first` the embedding's output as it was before the first layer
+    (float32 [T, H]; None unless the kind says `needs_first`)."""
+    needs_first = False
+
+    def forward(self, stream: "Stream", first: Optional[torch.Tensor], ctx: StepContext) -> "Stream":
         raise NotImplementedError
 
 
@@ -287,6 +318,7 @@ POSITION_ENCODINGS: Dict[str, type] = {}
 BLOCKS: Dict[str, type] = {}
 EMBEDDINGS: Dict[str, type] = {}
 HEADS: Dict[str, type] = {}
+STREAM_OPS: Dict[str, type] = {}
 
 
 def _register(table: Dict[str, type], what: str) -> Callable[[str], Callable[[type], type]]:
@@ -306,6 +338,7 @@ register_position_encoding = _register(POSITION_ENCODINGS, "position encoding")
 register_block = _register(BLOCKS, "block")
 register_embedding = _register(EMBEDDINGS, "embedding")
 register_head = _register(HEADS, "head")
+register_stream_op = _register(STREAM_OPS, "stream op")
 
 
 def _lookup(table: Dict[str, type], what: str, kind: str) -> type:
@@ -341,3 +374,7 @@ def embedding_class(kind: str) -> type:
 
 def head_class(kind: str) -> type:
     return _lookup(HEADS, "head", kind)
+
+
+def stream_op_class(kind: str) -> type:
+    return _lookup(STREAM_OPS, "stream op", kind)

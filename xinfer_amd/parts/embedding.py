@@ -3,6 +3,10 @@
 "embedding": x = E[ids] (times `scale` if the spec gives one; Qwen3 gives none) into the
 float32 residual stream; with `sinusoid_base` b a sinusoidal position vector is added, entry 2i =
 sin(p b^(-2i / dim)), entry 2i + 1 = cos of the same angle, for the token's position p (float32) (reference: /root/reference/src/models/qwen3.rs:211-220,302-309).
+With `pairs` (name, buckets, mul_prev, mul_cur) a row of a second table [buckets + 1, dim] is added, chosen by the
+token and the one before it: row (prev * mul_prev + token * mul_cur) mod buckets, and the last row for a sequence's
+first token.  The token before is state of the request: the embedding keeps one int32 a live request
+(`state_need`), written after every step, so a prompt may be cut anywhere.
 "lm_head": logits = h @ W^T in float32; W is the embedding table when the spec says `tied`
 (qwen3.rs:267-287,367-373); `scale` s, if the spec gives one, multiplies them; `softcap` c, if the spec
 gives one, then makes them c * tanh(logits / c).
@@ -16,7 +20,7 @@ import torch
 from .. import kernels
 from ..config.spec import PartSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import Head, StepContext, TokenEmbedding, register_embedding, register_head
+from .base import Head, LayerCache, StateNeed, StepContext, TokenEmbedding, register_embedding, register_head
 from .linear import Linear
 
 
@@ -33,21 +37,45 @@ class Embedding(TokenEmbedding):
         self.freq: Optional[torch.Tensor] = None      # float32 [(dim + 1) / 2]: base^(-2i / dim)
         self.rows: Optional[torch.Tensor] = None      # the last step's result rounded to the activation dtype
         self.table: Optional[torch.Tensor] = None
+        pairs = spec.get("pairs")
+        self.pairs = None if not pairs else dict(name=str(pairs["name"]), buckets=int(pairs["buckets"]),
+                                                 mul_prev=int(pairs["mul_prev"]), mul_cur=int(pairs["mul_cur"]))
+        if self.pairs is not None and (self.pairs["buckets"] <= 0 or min(self.pairs["mul_prev"], self.pairs["mul_cur"]) < 0):
+            raise ValueError("an embedding of pairs needs buckets and multipliers that are not negative")
+        if self.pairs is not None and self.sinusoid_base > 0:
+            raise NotImplementedError("an embedding with sinusoidal positions and a table of pairs")
+        self.pair_table: Optional[torch.Tensor] = None
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str = "") -> List[TensorDecl]:
-        return [TensorDecl(spec["name"], (int(spec["vocab_size"]), int(spec["dim"])))]
+        out = [TensorDecl(spec["name"], (int(spec["vocab_size"]), int(spec["dim"])))]
+        if spec.get("pairs"):
+            out.append(TensorDecl(spec["pairs"]["name"], (int(spec["pairs"]["buckets"]) + 1, int(spec["dim"]))))
+        return out
+
+    def state_need(self) -> Optional[StateNeed]:
+        return StateNeed((), torch.int32, "last_token") if self.pairs is not None else None
 
     def load(self, store: WeightStore, prefix: str, device) -> None:
         t = store.get(self.spec["name"], None, device)
         if self.dtype == torch.float32 or t.dtype != torch.float32:
             t = t.to(self.dtype)
         self.table = t.contiguous()
+        if self.pairs is not None:
+            self.pair_table = store.get(self.pairs["name"], None, device).to(self.table.dtype).contiguous()
         if self.sinusoid_base > 0:
             i = torch.arange((self.dim + 1) // 2, dtype=torch.float32)
             self.freq = (torch.tensor(self.sinusoid_base, dtype=torch.float32) ** (-2.0 * i / self.dim)).to(device).contiguous()
 
-    def forward(self, ids: torch.Tensor, ctx: Optional[StepContext] = None) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, ctx: Optional[StepContext] = None, cache: Optional[LayerCache] = None) -> torch.Tensor:
+        if self.pairs is not None:
+            if ctx is None or cache is None or cache.state is None:
+                raise ValueError("an embedding of pairs needs the step and its slots of the tokens before")
+            p = self.pairs
+            out = kernels.embed_pair(self.table, self.pair_table, ids, ctx.positions, ctx.tok_seq, ctx.cu_q, ctx.state_slots,
+                                     cache.state, self.scale, p["buckets"], p["mul_prev"], p["mul_cur"])
+            kernels.keep_last_token(ids, ctx.cu_q, ctx.state_slots, cache.state)
+            return out
         if self.freq is None:
             return kernels.embed(self.table, ids, scale=self.scale)
         if ctx is None:

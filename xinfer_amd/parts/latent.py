@@ -1,0 +1,118 @@
+"""Attention over a cached latent, as a mixer: "latent_attention".
+
+    q = W_q h                          heads of [dim plain | rot_dim turned] dims
+    down = W_dkv h                     rank + rot_dim rows: c = RMSNorm(down[:rank]) * w, and down[rank:], turned by the
+                                       token's position, is one key part shared by all heads
+    head i: k = [U_k,i c | turned part], v = U_v,i c
+    score = (q_plain . U_k,i c + q_turned . k_turned) * scale over the last `window` tokens (0: all)
+    softmax, with exp(sink_i) in its denominator if the spec says `sinks`
+    o = W_o (heads * sigmoid(W_g h))   (the gate only if the spec says `gate`)
+
+What a token keeps in the cache is c and the turned key part: one pool "latent" [pages, 1, page, rank + rot_dim].  The
+heads' matrices move to the query's side: q' = [U_k,i^T q_plain | q_turned] is scored against the cached rows directly,
+the weighted sum of the cached c is taken once a head, and U_v,i is applied to that sum; a token's keys and values are
+never made.  The gate is applied where U_v's product is stored.  Rotation tables, the latent's norm, scores, softmax and
+sinks are float32 in both precisions.  Tensor names under the part's prefix: q, dkv, dkv.norm, uk, uv, sink, g, o (the
+spec's `names` replaces any).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels
+from ..config.spec import PartSpec
+from ..weights.store import TensorDecl, WeightStore
+from .base import KVNeed, LayerCache, Mixer, PAGE, PoolNeed, StepContext, position_encoding_class, register_mixer
+from .linear import Linear
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    graph_safe = True
+    NAMES: Dict[str, str] = {"q": "q", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "sink": "sink",
+                             "g": "g", "o": "o"}
+
+    def __init__(self, spec: PartSpec, dtype: torch.dtype):
+        super().__init__(spec, dtype)
+        self.hidden = int(spec["hidden_size"])
+        self.heads = int(spec["num_heads"])
+        self.d = int(spec["head_dim"])              # plain dims of a head's q and k
+        self.r = int(spec["rot_dim"])               # turned dims
+        self.dv = int(spec["value_dim"])
+        self.rank = int(spec["kv_rank"])
+        self.scale = float(spec["scale"])
+        self.window = int(spec.get("window") or 0)
+        self.eps = float(spec["norm_eps"])
+        self.has_sinks = bool(spec.get("sinks", False))
+        self.has_gate = bool(spec.get("gate", False))
+        if min(self.hidden, self.heads, self.d, self.dv, self.rank) <= 0 or self.r <= 0 or self.r % 2:
+            raise ValueError(f"{self.heads} heads of {self.d} + {self.r} dims with values of {self.dv} over a latent of "
+                             f"{self.rank} cannot be run")
+        pos = spec.get("position")
+        if pos is None or int(pos.get("rotary_dim", pos["head_dim"])) != self.r:
+            raise ValueError("latent attention turns the whole of its rot_dim dims: it needs a position encoding of that size")
+        self.position = position_encoding_class(pos.kind)(pos, dtype)
+        self.proj: Optional[Linear] = None          # [q | dkv | g] rows
+        self.o: Optional[Linear] = None
+        self.uk = self.uv = None                    # [heads, dim, rank] and [heads, vdim, rank], as stored
+        self.norm_w = self.sinks = None
+
+    @classmethod
+    def _names(cls, spec: PartSpec, prefix: str) -> Dict[str, str]:
+        given = spec.get("names") or {}
+        return {k: f"{prefix}.{given.get(k, v)}" for k, v in cls.NAMES.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
+        h, H, d, r, dv, rank = (int(spec[k]) for k in ("hidden_size", "num_heads", "head_dim", "rot_dim", "value_dim", "kv_rank"))
+        n = cls._names(spec, prefix)
+        out = [TensorDecl(n["q"], (H * (d + r), h)), TensorDecl(n["dkv"], (rank + r, h)), TensorDecl(n["dkv_norm"], (rank,), "norm"),
+               TensorDecl(n["uk"], (H * d, rank)), TensorDecl(n["uv"], (H * dv, rank)), TensorDecl(n["o"], (h, H * dv))]
+        if spec.get("sinks", False):
+            out.append(TensorDecl(n["sink"], (H,), "normal(0,1)"))
+        if spec.get("gate", False):
+            out.append(TensorDecl(n["g"], (H * dv, h)))
+        return out
+
+    def _lin(self, store: WeightStore, name: str, device) -> torch.Tensor:
+        t = store.get(name, None, device)
+        return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
+
+    def load(self, store: WeightStore, prefix: str, device) -> None:
+        n = self._names(self.spec, prefix)
+        parts = [self._lin(store, n[k], device) for k in (("q", "dkv", "g") if self.has_gate else ("q", "dkv"))]
+        self.proj = Linear(torch.cat([p.to(self.dtype) for p in parts], dim=0))
+        self.o = Linear(self._lin(store, n["o"], device).to(self.dtype))
+        self.uk = self._lin(store, n["uk"], device).to(self.dtype).contiguous().view(self.heads, self.d, self.rank)
+        self.uv = self._lin(store, n["uv"], device).to(self.dtype).contiguous().view(self.heads, self.dv, self.rank)
+        self.norm_w = store.get(n["dkv_norm"], torch.float32, device).contiguous()
+        if self.has_sinks:
+            self.sinks = store.get(n["sink"], torch.float32, device).contiguous()
+        self.position.load(store, prefix, device)
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.window, (PoolNeed("latent", (1, PAGE, self.rank + self.r)),))
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        H, d, r, dv, rank = self.heads, self.d, self.r, self.dv, self.rank
+        T = x.shape[0]
+        p = self.proj(x, out_dtype=self.dtype)
+        q_cols, down_at = H * (d + r), H * (d + r)
+        pool = cache.pools["latent"]
+        slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
+        pos = self.position
+        q_full = torch.empty((T, H, rank + r), dtype=self.dtype, device=x.device)
+        kernels.latent_rows(p, 0, down_at, self.norm_w, self.eps, slots, pool, q_full, H, d, r, rank, pos.cos, pos.sin,
+                            pos.interleaved, ctx.positions)
+        # the plain part of every head's query through its U_k: out[t, h, j] = sum_i q[t, h, i] U_k[h, i, j]
+        q_plain = p[:, :q_cols].view(T, H, d + r)[:, :, :d]
+        kernels.head_linear(q_plain, self.uk.transpose(1, 2), q_full[:, :, :rank])
+        a = kernels.attention_generic(q_full, pool, None, ctx.block_tables[cache.group], ctx.tok_seq, ctx.positions, self.scale,
+                                      self.window, sinks=self.sinks, value_dim=rank)
+        # the heads' weighted sums of the latent through their U_v, times the gate
+        heads = torch.empty((T, H, dv), dtype=self.dtype, device=x.device)
+        gate = p[:, q_cols + rank + r:].view(T, H, dv) if self.has_gate else None
+        kernels.head_linear(a.view(T, H, rank), self.uv, heads, gate=gate)
+        return self.o(heads.view(T, H * dv), out_dtype=self.dtype, allow_split=True)

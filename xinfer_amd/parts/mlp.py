@@ -66,3 +66,44 @@ class GatedMLP(FeedForward):
         elif m is None:
             m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))
         return self.down(m, out_dtype=self.dtype, allow_split=True, sink=sink)   # the next norm adds the parts
+
+
+@register_feed_forward("mlp")
+class DenseMLP(FeedForward):
+    """Feed-forward without a gate: down(act(up(x))), act one of `kernels.UNGATED_ACTIVATIONS` (silu, the tanh form
+    of gelu, or relu2: the square of relu).  Tensor names as data (`names`: up, down)."""
+    graph_safe = True
+    NAMES = {"up": "up_proj.weight", "down": "down_proj.weight"}
+
+    def __init__(self, spec: PartSpec, dtype: torch.dtype):
+        super().__init__(spec, dtype)
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.activation = str(spec.get("activation", "relu2"))
+        if self.activation not in kernels.UNGATED_ACTIVATIONS:
+            raise NotImplementedError(f"activation {self.activation!r} is not built ({', '.join(kernels.UNGATED_ACTIVATIONS)})")
+        self.up: Optional[Linear] = None
+        self.down: Optional[Linear] = None
+
+    @classmethod
+    def _names(cls, spec: PartSpec, prefix: str):
+        given = spec.get("names") or {}
+        return {k: f"{prefix}.{given.get(k, v)}" for k, v in cls.NAMES.items()}
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
+        h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
+        n = cls._names(spec, prefix)
+        return [TensorDecl(n["up"], (i, h)), TensorDecl(n["down"], (h, i))]
+
+    def load(self, store: WeightStore, prefix: str, device) -> None:
+        def lin(name):
+            t = store.get(name, None, device)
+            return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
+        n = self._names(self.spec, prefix)
+        self.up = Linear(lin(n["up"]))
+        self.down = Linear(lin(n["down"]))
+
+    def forward(self, x, ctx: StepContext):
+        m = kernels.act_(self.up(x, out_dtype=self.dtype), self.activation)
+        return self.down(m, out_dtype=self.dtype, allow_split=True)      # the next norm adds the parts

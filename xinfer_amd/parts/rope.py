@@ -111,6 +111,21 @@ def scaled_inv_freq(theta: float, rot: int, scaling) -> "tuple[np.ndarray, float
         inv = (inter * (f32(1.0) - mask) + extra * mask).astype(f32)
         mscale = f32(1.0) if factor <= 1.0 else f32(0.1) * f32(1.0) * np.log(factor) + f32(1.0)
         return inv, float(f32(mscale * f32(scaling["attn_factor"])))
+    if kind == "ramp":
+        # Frequencies blended along a ramp over the pair index: with dim(t) = rot ln(original / (2 pi t)) / (2 ln theta),
+        # lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001),
+        # 0, 1), frequency i is f_i / factor * r_i + f_i (1 - r_i), and cos and sin grow by 0.1 ln(factor) + 1.  Made in
+        # float64 and rounded once.
+        factor = float(scaling["factor"])
+        f = np.power(np.float64(theta), -np.arange(0, rot, 2, dtype=np.float64) / rot)
+
+        def dim_of(turns: float) -> float:
+            return rot * math.log(orig / (2.0 * math.pi * float(turns))) / (2.0 * math.log(theta))
+
+        lo = max(math.floor(dim_of(scaling["fast"])), 0)
+        hi = min(math.ceil(dim_of(scaling["slow"])), rot - 1)
+        ramp = np.clip((np.arange(rot // 2, dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return (f / factor * ramp + f * (1.0 - ramp)).astype(f32), 0.1 * math.log(factor) + 1.0
     raise ValueError(f"Unknown rope_type: {kind}")
 
 

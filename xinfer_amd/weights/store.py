@@ -58,7 +58,7 @@ class WeightError(RuntimeError):
 class TensorDecl:
     """A tensor a part needs.  `init` names how random weights fill it:
     "linear" ~ N(0, linear_std), "norm" ~ 1 + N(0, norm_std), "mix" ~ 0.5 + N(0, norm_std) (a blend's
-    scalar), "zeros"."""
+    scalar), "zeros", "normal(shift,scale)" ~ shift + N(0, scale) with the two numbers written out."""
     name: str
     shape: Tuple[int, ...]
     init: str = "linear"
@@ -197,6 +197,8 @@ class RandomStore(WeightStore):
             scale, shift = self.norm_std, 0.5
         elif d.init == "linear":
             scale, shift = self.linear_std, 0.0
+        elif d.init.startswith("normal(") and d.init.endswith(")"):
+            shift, scale = (float(v) for v in d.init[7:-1].split(","))
         else:
             raise ValueError(f"tensor {name!r}: unknown init {d.init!r}")
         key = self._tensor_key(name)
