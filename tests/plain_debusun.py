@@ -95,38 +95,56 @@ def window_softmax(scores, window, sink=None):
     return e / den
 
 
+def _window(m):
+    return m["mask"]["size"] if m.get("mask") else 1 << 30
+
+
 # ---- the three mixers ------------------------------------------------------------------------------------
+def attention_heads(q, k, v, m, eps, positions):
+    """q [T, H, d], k [T, G, d], v [T, G, dv] as projected: rotation, then each q and k head divided by its root mean
+    square, scores times scale over the window, softmax; query head i reads kv head i // (H / G).  Returns [T, H dv]."""
+    T, H, _ = q.shape
+    G, dv = k.shape[1], v.shape[2]
+    if m.get("rot"):
+        q, k = rotate(q, m["rot"], positions), rotate(k, m["rot"], positions)
+    q, k = rms_norm(q, eps), rms_norm(k, eps)
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
+    for hd in range(H):
+        g = hd // (H // G)
+        p = window_softmax((q[:, hd] @ k[:, g].T) * m["scale"], _window(m))
+        out[:, hd] = p @ v[:, g]
+    return out.reshape(T, H * dv)
+
+
 def attention(h, w, m, eps, positions):
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     T = h.shape[0]
-    q = rotate((h @ w["q"].T).view(T, H, d), m["rot"], positions)
-    k = rotate((h @ w["k"].T).view(T, G, d), m["rot"], positions)
-    v = (h @ w["v"].T).view(T, G, dv)
-    q, k = rms_norm(q, eps), rms_norm(k, eps)
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
-    for hd in range(H):
-        g = hd // (H // G)
-        p = window_softmax((q[:, hd] @ k[:, g].T) * m["scale"], m["mask"]["size"])
-        out[:, hd] = p @ v[:, g]
-    return out.reshape(T, H * dv) @ w["o"].T
+    heads = attention_heads((h @ w["q"].T).view(T, H, d), (h @ w["k"].T).view(T, G, d), (h @ w["v"].T).view(T, G, dv), m, eps,
+                            positions)
+    return heads @ w["o"].T
 
 
-def latent_attention(h, w, m, eps, positions):
+def latent_heads(q, down, w, m, eps, positions):
+    """q [T, H, d + r] and down [T, rank + r] as projected; w holds dkv.norm, uk, uv, sink.  Returns the heads
+    [T, H dv] before the gate."""
     H, d, r, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
-    T = h.shape[0]
-    q = (h @ w["q"].T).view(T, H, d + r)
+    T = q.shape[0]
     q_plain, q_turned = q[..., :d], rotate(q[..., d:], m["rot"], positions)
-    down = h @ w["dkv"].T
     c = rms_norm(down[:, :rank], eps, w["dkv.norm"])
     k_turned = rotate(down[:, None, rank:], m["rot"], positions)[:, 0]          # one part for all heads
     k_plain = (c @ w["uk"].T).view(T, H, d)
     v = (c @ w["uv"].T).view(T, H, dv)
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
     for hd in range(H):
         s = (q_plain[:, hd] @ k_plain[:, hd].T + q_turned[:, hd] @ k_turned.T) * m["scale"]
-        out[:, hd] = window_softmax(s, m["mask"]["size"], sink=w["sink"][hd]) @ v[:, hd]
-    gate = torch.sigmoid(h @ w["g"].T)
-    return (out.reshape(T, H * dv) * gate) @ w["o"].T
+        out[:, hd] = window_softmax(s, _window(m), sink=w["sink"][hd]) @ v[:, hd]
+    return out.reshape(T, H * dv)
+
+
+def latent_attention(h, w, m, eps, positions):
+    T = h.shape[0]
+    heads = latent_heads((h @ w["q"].T).view(T, m["heads"], m["dim"] + m["rot_dim"]), h @ w["dkv"].T, w, m, eps, positions)
+    return (heads * torch.sigmoid(h @ w["g"].T)) @ w["o"].T
 
 
 def causal_conv(u, taps_w, bias):
@@ -140,6 +158,29 @@ def causal_conv(u, taps_w, bias):
     return out
 
 
+def state_space(x, B, C, dt, decay_log, skip, state=None):
+    """x [T, H, dv], B and C [T, G, N], dt [T, H] (step sizes, after the softplus): per head i (group i // (H / G))
+    S <- exp(-exp(decay_log_i) dt) S + dt B x^T, y = S^T C + skip_i x.  Returns (y [T, H, dv], the last S [H, N, dv])."""
+    T, H, dv = x.shape
+    G, N = B.shape[1], B.shape[2]
+    decay = torch.exp(-torch.exp(decay_log)[None, :] * dt)                     # [T, H]
+    y = torch.zeros(T, H, dv, dtype=x.dtype)
+    S = torch.zeros(H, N, dv, dtype=x.dtype) if state is None else state.clone()
+    for hd in range(H):
+        g = hd // (H // G)
+        for t in range(T):
+            S[hd] = decay[t, hd] * S[hd] + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
+            y[t, hd] = S[hd].T @ C[t, g] + skip[hd] * x[t, hd]
+    return y, S
+
+
+def gated_group_norm(y, z, weight, eps, parts):
+    """y, z [T, inner]: y * silu(z), each of `parts` equal parts of a row divided by its root mean square, times weight."""
+    T, inner = y.shape
+    y = y * silu(z)
+    return rms_norm(y.view(T, parts, inner // parts), eps).reshape(T, inner) * weight
+
+
 def mamba2(h, w, m, eps):
     H, dv, N, G, parts = m["heads"], m["vdim"], m["state"], m["groups"], m["norm_groups"]
     inner = H * dv
@@ -150,18 +191,8 @@ def mamba2(h, w, m, eps):
     x = xbc[:, :inner].view(T, H, dv)
     B = xbc[:, inner:inner + G * N].view(T, G, N)
     C = xbc[:, inner + G * N:].view(T, G, N)
-    dt = softplus(dt + w["dt_bias"])
-    decay = torch.exp(-torch.exp(w["A_log"])[None, :] * dt)                     # [T, H]
-    y = torch.zeros(T, H, dv, dtype=h.dtype)
-    for hd in range(H):
-        g = hd // (H // G)
-        S = torch.zeros(N, dv, dtype=h.dtype)
-        for t in range(T):
-            S = decay[t, hd] * S + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
-            y[t, hd] = S.T @ C[t, g] + w["D"][hd] * x[t, hd]
-    y = y.reshape(T, inner) * silu(z)
-    y = rms_norm(y.view(T, parts, inner // parts), eps).reshape(T, inner) * w["norm"]
-    return y @ w["o"].T
+    y, _ = state_space(x, B, C, softplus(dt + w["dt_bias"]), w["A_log"], w["D"])
+    return gated_group_norm(y.reshape(T, inner), z, w["norm"], eps, parts) @ w["o"].T
 
 
 def dense_mlp(h, w):
@@ -228,3 +259,9 @@ class PlainDebusun:
     def logits(self, tokens):
         x = self.stream(tokens)[-1]
         return rms_norm(x, self.cfg["norm"]["eps"], self.w["final.norm"]) @ self.w["head"].T
+
+    def greedy(self, prompt, n):
+        ids = list(prompt)
+        for _ in range(n):
+            ids.append(int(self.logits(ids)[-1].argmax()))
+        return ids[len(prompt):]
