@@ -43,8 +43,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale,
-    float softcap, const float* __restrict__ slopes, int window, int page_shift, int nq, int nkv, int d, int dv,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits) {
+    float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks, int window, int page_shift, int nq,
+    int nkv, int d, int dv, float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits) {
   const int page = 1 << page_shift;
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
@@ -349,6 +349,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
       }
       continue;
     }
+    // a sink: one more weight in the denominator, exp(sink) on the scale of the reference point, with no value
+    if (sinks) lt += __builtin_amdgcn_exp2f(sinks[h0 + hh] * kLog2eB - m_run[ct]);
     const float inv = 1.f / lt;
     bf16* o = out + ((size_t)(q_begin + qi) * nq + h0 + hh) * dv;
 #pragma unroll
@@ -368,8 +370,10 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
 // order (m_s: the slice's reference point in the exponent's unit; a slice without keys has m_s = -inf).
 __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml, bf16* __restrict__ out,
-                                                                 int max_splits, int nq, int dv) {
+                                                                 const float* __restrict__ sinks, int max_splits, int nq,
+                                                                 int dv) {
   const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const float sink2 = sinks ? sinks[head] * kLog2eB : -INFINITY;      // the head's sink in the exponent's unit
   const size_t base = ((size_t)t * nq + head) * max_splits;
   __shared__ float f_s[64];
   if (max_splits <= 64) {          // a slice a lane: one round of loads for the weights, one for the sums
@@ -381,7 +385,7 @@ __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __
     }
     const float mm = wave_max(ms);
     const float f = ms > -INFINITY ? __builtin_amdgcn_exp2f(ms - mm) : 0.f;
-    const float inv = 1.f / wave_sum(ls * f);
+    const float inv = 1.f / (wave_sum(ls * f) + (sinks ? __builtin_amdgcn_exp2f(sink2 - mm) : 0.f));
     f_s[lane] = f;
     __syncthreads();
     for (int i = lane; i < dv; i += 64) {
@@ -402,6 +406,7 @@ __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __
     const float ms = part_ml[(base + s2) * 2];
     if (ms > -INFINITY) ll += part_ml[(base + s2) * 2 + 1] * __builtin_amdgcn_exp2f(ms - mm);
   }
+  if (sinks) ll += __builtin_amdgcn_exp2f(sink2 - mm);
   const float inv = 1.f / ll;
   for (int i = lane; i < dv; i += 64) {
     float o = 0.f;
@@ -439,11 +444,11 @@ int xi_attention_biased_block(int d, int dv, int g, int small) {
 
 // tiles int32 [n_tiles, 2] = (sequence, first query position of the block within the sequence's portion).
 // q [T, nq, d]; K pool [pages, nkv, page, d]; V pool [pages, nkv, page / 8, dv, 8]; out [T, nq * dv].
-// softcap 0: none; slopes null: none.
+// softcap 0: none; slopes null: none; sinks null: none, else float32 [nq], exp(sinks[h]) joins head h's denominator.
 int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
                              int max_pages, const int* tiles, int n_tiles, const int* cu_q, const int* ctx_lens,
-                             void* out, float scale, float softcap, const float* slopes, int window, int page, int nq,
-                             int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
+                             void* out, float scale, float softcap, const float* slopes, const float* sinks, int window,
+                             int page, int nq, int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
                              int max_splits, int n_tok, hipStream_t stream) {
   XI_CHECK(xi_attention_biased_supported(nq, nkv, d, dv, page), "attention_biased: unsupported sizes nq=%d nkv=%d d=%d dv=%d page=%d",
            nq, nkv, d, dv, page);
@@ -477,8 +482,8 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
     }                                                                                                   \
     kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
                                           block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
-                                          scale, softcap, slopes, window, page_shift, nq, nkv, d, dv,   \
-                                          part_o, part_ml, split_keys, max_splits);                     \
+                                          scale, softcap, slopes, sinks, window, page_shift, nq, nkv, d,\
+                                          dv, part_o, part_ml, split_keys, max_splits);                 \
   } while (0)
 #define XI_PB_GH(KC, DT, NQT, NWV)             \
   do {                                         \
@@ -517,7 +522,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
 #undef XI_PB
   XI_LAUNCH_CHECK("attention_biased");
   if (split_keys > 0) {
-    attn_biased_combine_kernel<<<dim3(nq, n_tok), 64, 0, stream>>>(part_o, part_ml, (bf16*)out, max_splits, nq, dv);
+    attn_biased_combine_kernel<<<dim3(nq, n_tok), 64, 0, stream>>>(part_o, part_ml, (bf16*)out, sinks, max_splits, nq, dv);
     XI_LAUNCH_CHECK("attention_biased_combine");
   }
   return 0;

@@ -5,7 +5,8 @@
 //   score(i, j) = ((U_k^T q_plain_i) . c_j + q_turned_i . k_turned_j) * scale        o_i = U_v (sum_j p_ij c_j)
 //
 // so the attention itself is one kv head with keys [c | k_turned] of rank + r dims whose first `rank` dims are
-// the values too, read from one pool [pages, 1, page, rank + r].
+// the values too, read from one pool [pages, 1, page, rank + r].  The matrix-core attention kernels read values in
+// groups of eight keys, [pages, 1, page / 8, rank, 8]: where such a pool is given, c is written there once more.
 //
 // `latent_rows_kernel`, a workgroup a token, from the packed projection row [q (H (dim + r)) | down (rank + r) | ..]:
 //   c = down[:rank] / sqrt(mean(down[:rank]^2) + eps) * w   and the turned down[rank:] into the pool at the slot;
@@ -23,7 +24,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ proj, long long proj_stride, int q_off,
                                                           int down_off, const float* __restrict__ w, float eps,
                                                           const long long* __restrict__ slots, T* __restrict__ pool,
-                                                          int page_size, T* __restrict__ q_full, int H, int dim, int r,
+                                                          T* __restrict__ values, int page_size, T* __restrict__ q_full, int H, int dim, int r,
                                                           int rank, const float* __restrict__ cos_t,
                                                           const float* __restrict__ sin_t, int interleaved,
                                                           const int* __restrict__ positions) {
@@ -54,7 +55,15 @@ __global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ 
   const long long slot = slots[t];
   if (slot < 0) return;
   T* dst = pool + (size_t)slot * (rank + r);       // [pages, 1, page, rank + r]: slot = page * page_size + offset
-  for (int i = threadIdx.x; i < rank; i += blockDim.x) dst[i] = from_float<T>(to_float(down[i]) * inv * w[i]);
+  // values in groups of eight keys: token `off` of a page at [off / 8][i][off % 8]
+  const long long pg = slot / page_size;
+  const int off = (int)(slot - pg * page_size);
+  T* vdst = values ? values + ((size_t)pg * (page_size / 8) + off / 8) * (size_t)rank * 8 + (off & 7) : nullptr;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const T c = from_float<T>(to_float(down[i]) * inv * w[i]);
+    dst[i] = c;
+    if (vdst) vdst[(size_t)i * 8] = c;
+  }
   for (int p = threadIdx.x; p < half; p += blockDim.x) {
     const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
     const float a = to_float(down[rank + ia]), b = to_float(down[rank + ib]);
@@ -139,7 +148,7 @@ extern "C" {
 // proj rows of proj_stride elements: the heads' q parts [H, dim + r] from q_off, the down projection [rank + r] from
 // down_off; w float32 [rank]; pool [pages, 1, page, rank + r]; q_full [T, H, rank + r] (its last r dims are written).
 int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_off, int dtype, const float* w, float eps,
-                   const long long* slots, void* pool, int page_size, void* q_full, int n_tok, int H, int dim, int r, int rank,
+                   const long long* slots, void* pool, void* values, int page_size, void* q_full, int n_tok, int H, int dim, int r, int rank,
                    const float* cos_t, const float* sin_t, int interleaved, const int* positions, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && H > 0 && dim > 0 && r >= 0 && r % 2 == 0 && rank > 0 && page_size > 0,
            "latent_rows: bad sizes T=%d H=%d dim=%d r=%d rank=%d page=%d", n_tok, H, dim, r, rank, page_size);
@@ -148,14 +157,15 @@ int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_
            "latent_rows: the projection's rows are too short");
   XI_CHECK(r == 0 || (cos_t && sin_t), "latent_rows: a rotation needs its tables");
   XI_CHECK(w && positions && slots, "latent_rows: the norm's weight, the positions and the slots are needed");
+  XI_CHECK(values == nullptr || page_size % 8 == 0, "latent_rows: values in groups of eight need pages of a multiple of 8");
   if (n_tok == 0) return 0;
   if (dtype == kF32)
     latent_rows_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)proj, proj_stride, q_off, down_off, w, eps, slots,
-                                                         (float*)pool, page_size, (float*)q_full, H, dim, r, rank, cos_t,
+                                                         (float*)pool, (float*)values, page_size, (float*)q_full, H, dim, r, rank, cos_t,
                                                          sin_t, interleaved, positions);
   else if (dtype == kBF16)
     latent_rows_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)proj, proj_stride, q_off, down_off, w, eps, slots,
-                                                        (bf16*)pool, page_size, (bf16*)q_full, H, dim, r, rank, cos_t, sin_t,
+                                                        (bf16*)pool, (bf16*)values, page_size, (bf16*)q_full, H, dim, r, rank, cos_t, sin_t,
                                                         interleaved, positions);
   else
     XI_CHECK(false, "latent_rows: unknown dtype %d", dtype);

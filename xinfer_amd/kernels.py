@@ -1030,17 +1030,21 @@ def biased_split_keys(workgroups: int, span: int) -> int:
 
 
 def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, softcap=0.0,
-                          slopes=None, out=None, small=0, split_keys=0, span=0):
+                          slopes=None, out=None, small=0, split_keys=0, span=0, sinks=None):
     """Matrix-core attention for any mix of portions with the score's options (`softcap`, `slopes`: see
-    `attention_generic`) and a value head size of its own: q [T, nq, d], K pool [pages, nkv, page, d], V pool
+    `attention_generic`; `sinks` as there) and a value head size of its own: q [T, nq, d], K pool [pages, nkv, page, d], V pool
     [pages, nkv, page / 8, dv, 8]; tiles int32 [n, 2] = (sequence, first query token of a block of
     `attention_biased_block(d, dv, nq // nkv, small)` tokens within the sequence's portion).  Returns [T, nq * dv].
     `split_keys` > 0 (steps in which every sequence brings one token, a tile a token): each workgroup walks one slice
     of that many keys of the up to `span` a token sees, and a second kernel puts the slices together."""
-    _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes)
+    _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes, sinks)
     T, nq, d = q.shape
     nkv, page, dv = k_cache.shape[1], k_cache.shape[2], int(vt_cache.shape[3])
     _want(q, torch.bfloat16, "attention_biased: q")
+    if sinks is not None:
+        _want(sinks, torch.float32, "attention_biased: sinks")
+        if sinks.shape != (nq,):
+            raise KernelError(f"attention_biased: sinks {tuple(sinks.shape)} must be one a query head, [{nq}]")
     _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv)
     for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
         _want(t, torch.int32, f"attention_biased: {name}")
@@ -1069,8 +1073,8 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
         part_ml = torch.empty((T, nq, max_splits, 2), dtype=torch.float32, device=q.device)
     _ok(lib().xi_attention_biased_bf16(
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
-        _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), int(window), int(page),
-        nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), _stream()))
+        _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), _p(sinks), int(window),
+        int(page), nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), _stream()))
     return out
 
 
@@ -1161,17 +1165,22 @@ def attention_decode_packed_bf16(qkv, q_weight, k_weight, eps, cos, sin, rotary_
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
               scale: float, window: int = 0, v_grouped: bool = False, softcap: float = 0.0,
-              slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+              slopes: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None,
+              value_dim: Optional[int] = None) -> torch.Tensor:
     """Attention of one step's tokens over the paged cache of `group`; chooses the kernel
     from the precision and the shape of the batch: float32, or sizes the matrix-core
     kernels do not take, go to the generic kernel; bfloat16 batches of single tokens to
     the split-K decode kernel; everything else to the prefill kernel.  Scores with a soft cap
-    or a distance bias, and values of another head size than the keys, have matrix-core
-    kernels of their own (`attention_biased_bf16`)."""
+    or a distance bias, a softmax with sinks, and values of another head size than the keys, have
+    matrix-core kernels of their own (`attention_biased_bf16`).  `v_cache` None: a key's first
+    `value_dim` dims are its value, which only the generic kernel reads that way."""
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
     bt = ctx.block_tables[group]
-    if softcap > 0 or slopes is not None or v_cache.shape[3] != d:
+    if v_cache is None:
+        return attention_generic(q, k_cache, None, bt, ctx.tok_seq, ctx.positions, scale, window, softcap=softcap,
+                                 slopes=slopes, sinks=sinks, value_dim=value_dim)
+    if softcap > 0 or slopes is not None or sinks is not None or v_cache.shape[3] != d:
         dv = int(v_cache.shape[3])
         if q.dtype == torch.bfloat16 and v_grouped and BIASED_MFMA and attention_biased_supported(nq, nkv, d, dv, page):
             key = ("attention_biased_tiles", d, dv, nq, nkv)
@@ -1193,9 +1202,9 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
                 span = min(int(ctx.max_ctx_len), int(window) + 63) if window > 0 else int(ctx.max_ctx_len)
                 split = biased_split_keys(ctx.num_seqs * nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1)), span)
             return attention_biased_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
-                                         softcap=softcap, slopes=slopes, small=small, split_keys=split, span=span)
+                                         softcap=softcap, slopes=slopes, small=small, split_keys=split, span=span, sinks=sinks)
         return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
-                                 v_grouped=v_grouped, softcap=softcap, slopes=slopes)
+                                 v_grouped=v_grouped, softcap=softcap, slopes=slopes, sinks=sinks)
     if q.dtype == torch.bfloat16 and v_grouped and mfma_attention_supported(nq, nkv, d, page):
         g = nq // nkv
         if ctx.max_q_len == 1 and decode_attention_takes(nq, nkv, d):
@@ -1719,12 +1728,14 @@ def head_rows(qkv: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_c
 # ---- attention over a latent ---------------------------------------------------------------------------------
 def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight: torch.Tensor, eps: float,
                 slots: torch.Tensor, pool: torch.Tensor, q_full: torch.Tensor, heads: int, dim: int, rot_dim: int,
-                rank: int, cos: torch.Tensor, sin: torch.Tensor, interleaved: bool, positions: torch.Tensor) -> None:
+                rank: int, cos: torch.Tensor, sin: torch.Tensor, interleaved: bool, positions: torch.Tensor,
+                values: Optional[torch.Tensor] = None) -> None:
     """From the packed projection `proj` [T, W] (the heads' q parts [H, dim + rot_dim] from column `q_offset`, the down
     projection [rank + rot_dim] from `down_offset`): the latent = RMSNorm(down[:rank]) * norm_weight and the turned
     down[rank:] into `pool` [pages, 1, page, rank + rot_dim] at `slots`; every head's turned q part into
-    q_full[:, h, rank:] (q_full [T, H, rank + rot_dim])."""
-    _dev(proj, norm_weight, slots, pool, q_full, cos, sin, positions)
+    q_full[:, h, rank:] (q_full [T, H, rank + rot_dim]).  `values` [pages, 1, page / 8, rank, 8]: the latent once
+    more, in groups of eight tokens, as the matrix-core attention kernels read values."""
+    _dev(proj, norm_weight, slots, pool, q_full, cos, sin, positions, values)
     H, d, r, rank = int(heads), int(dim), int(rot_dim), int(rank)
     if proj.dim() != 2 or q_full.dtype != proj.dtype or pool.dtype != proj.dtype:
         raise KernelError("latent_rows: the projection, the pool and q of one type")
@@ -1741,8 +1752,11 @@ def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight
     if (norm_weight.shape != (rank,) or slots.shape != (T,) or positions.shape != (T,) or r % 2 or cos.shape != sin.shape
             or cos.dim() != 2 or cos.shape[1] != r // 2):
         raise KernelError(f"latent_rows: weight [{rank}], slots and positions [T], tables [positions, {r // 2}]")
+    if values is not None and (values.dtype != proj.dtype or pool.shape[2] % 8
+                               or tuple(values.shape) != (pool.shape[0], 1, pool.shape[2] // 8, rank, 8)):
+        raise KernelError(f"latent_rows: the values' pool {tuple(values.shape)} must be [{pool.shape[0]}, 1, page / 8, {rank}, 8]")
     _ok(lib().xi_latent_rows(_p(proj), ctypes.c_longlong(W), int(q_offset), int(down_offset), _code(proj, "latent_rows"),
-                             _p(norm_weight), ctypes.c_float(eps), _p(slots), _p(pool), int(pool.shape[2]), _p(q_full), T, H,
+                             _p(norm_weight), ctypes.c_float(eps), _p(slots), _p(pool), _p(values), int(pool.shape[2]), _p(q_full), T, H,
                              d, r, rank, _p(cos), _p(sin), int(bool(interleaved)), _p(positions), _stream()))
 
 

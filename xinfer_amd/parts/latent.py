@@ -12,7 +12,11 @@ What a token keeps in the cache is c and the turned key part: one pool "latent" 
 heads' matrices move to the query's side: q' = [U_k,i^T q_plain | q_turned] is scored against the cached rows directly,
 the weighted sum of the cached c is taken once a head, and U_v,i is applied to that sum; a token's keys and values are
 never made.  The gate is applied where U_v's product is stored.  Rotation tables, the latent's norm, scores, softmax and
-sinks are float32 in both precisions.  Tensor names under the part's prefix: q, dkv, dkv.norm, uk, uv, sink, g, o (the
+sinks are float32 in both precisions.  In bfloat16, where the matrix-core attention kernel takes the sizes (rank + rot_dim
+up to 256, both multiples of 8), a second pool "latent_t" [pages, 1, page / 8, rank, 8] holds c once more, in the groups
+of eight tokens that kernel reads values in: portions and single tokens then run on the matrix cores, with one kv head
+of rank + rot_dim dims and values of rank dims; other sizes, and float32, read keys and values from the one pool
+with the generic kernel.  Tensor names under the part's prefix: q, dkv, dkv.norm, uk, uv, sink, g, o (the
 spec's `names` replaces any).
 """
 from __future__ import annotations
@@ -24,7 +28,7 @@ import torch
 from .. import kernels
 from ..config.spec import PartSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import KVNeed, LayerCache, Mixer, PAGE, PoolNeed, StepContext, position_encoding_class, register_mixer
+from .base import KVNeed, LayerCache, Mixer, PAGE, PAGE_BY_8, PoolNeed, StepContext, position_encoding_class, register_mixer
 from .linear import Linear
 
 
@@ -54,6 +58,10 @@ class LatentAttention(Mixer):
         if pos is None or int(pos.get("rotary_dim", pos["head_dim"])) != self.r:
             raise ValueError("latent attention turns the whole of its rot_dim dims: it needs a position encoding of that size")
         self.position = position_encoding_class(pos.kind)(pos, dtype)
+        # values in groups of eight tokens beside the keys: what the matrix-core kernel reads (any page it is given
+        # is a power of two of at least 8 where the engine runs bfloat16 attention on the matrix cores)
+        self.values_pool = (dtype == torch.bfloat16 and spec.get("matrix_cores", True)
+                            and kernels.attention_biased_supported(self.heads, 1, self.rank + self.r, self.rank, 64))
         self.proj: Optional[Linear] = None          # [q | dkv | g] rows
         self.o: Optional[Linear] = None
         self.uk = self.uv = None                    # [heads, dim, rank] and [heads, vdim, rank], as stored
@@ -93,7 +101,10 @@ class LatentAttention(Mixer):
         self.position.load(store, prefix, device)
 
     def cache_need(self) -> KVNeed:
-        return KVNeed(self.window, (PoolNeed("latent", (1, PAGE, self.rank + self.r)),))
+        pools = [PoolNeed("latent", (1, PAGE, self.rank + self.r))]
+        if self.values_pool:
+            pools.append(PoolNeed("latent_t", (1, PAGE_BY_8, self.rank, 8)))
+        return KVNeed(self.window, tuple(pools))
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         H, d, r, dv, rank = self.heads, self.d, self.r, self.dv, self.rank
@@ -101,16 +112,19 @@ class LatentAttention(Mixer):
         p = self.proj(x, out_dtype=self.dtype)
         q_cols, down_at = H * (d + r), H * (d + r)
         pool = cache.pools["latent"]
+        values = cache.pools.get("latent_t")
+        if values is not None and not kernels.attention_biased_supported(H, 1, rank + r, rank, pool.shape[2]):
+            values = None                                           # a page the matrix-core kernel does not take
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
         pos = self.position
         q_full = torch.empty((T, H, rank + r), dtype=self.dtype, device=x.device)
         kernels.latent_rows(p, 0, down_at, self.norm_w, self.eps, slots, pool, q_full, H, d, r, rank, pos.cos, pos.sin,
-                            pos.interleaved, ctx.positions)
+                            pos.interleaved, ctx.positions, values=values)
         # the plain part of every head's query through its U_k: out[t, h, j] = sum_i q[t, h, i] U_k[h, i, j]
         q_plain = p[:, :q_cols].view(T, H, d + r)[:, :, :d]
         kernels.head_linear(q_plain, self.uk.transpose(1, 2), q_full[:, :, :rank])
-        a = kernels.attention_generic(q_full, pool, None, ctx.block_tables[cache.group], ctx.tok_seq, ctx.positions, self.scale,
-                                      self.window, sinks=self.sinks, value_dim=rank)
+        a = kernels.attention(q_full, pool, values, ctx, cache.group, self.scale, self.window, v_grouped=values is not None,
+                              sinks=self.sinks, value_dim=rank)
         # the heads' weighted sums of the latent through their U_v, times the gate
         heads = torch.empty((T, H, dv), dtype=self.dtype, device=x.device)
         gate = p[:, q_cols + rank + r:].view(T, H, dv) if self.has_gate else None
