@@ -39,6 +39,9 @@ prefill of one prompt and a decode step at batch 8, one JSON line with both.
 `--design lilalorn[:SIZE]` times the Lilalorn family (layers of softmax attention beside retention, and of
 gated linear attention, in turn; experts without a gate and a shared one) beside the closest family there
 is, Mufenex with routed experts and no window, at equal sizes.
+`--design debusun[:SIZE]` times the Debusun family (layers of attention over a latent with sinks and a gate, of
+windowed attention whose heads are normed after the rotation, and of a selective state space, in turn; dense
+feed-forwards of a squared relu; a table of token pairs beside the embedding) beside dense Mufenex at equal sizes.
 """
 from __future__ import annotations
 
@@ -85,6 +88,13 @@ DESIGN_SIZES = {
     "1k-moe": dict(width=1024, heads=16, kv_heads=8, dim=128, vdim=128, ff=3072, window=1024, experts=8, top=2),
 }
 LILALORN_SIZES = ("1k-moe", "4k-moe", "2k-v")      # the sizes with experts: every Lilalorn layer has them
+DEBUSUN_SIZES = ("1k", "4k")                        # the dense sizes: every Debusun feed-forward is dense
+# Debusun's own sizes at every width: the latent and its turned part (together what the matrix-core kernel takes for
+# one head), the state space's head and state sizes (its inner width is twice the model's)
+DEBUSUN_LATENT = dict(kv_rank=192, rot_dim=64)
+DEBUSUN_STATE = dict(vdim=64, state=128, groups=1, conv=4, norm_groups=1)
+DESIGN_CHOICES = {"mufenex": (tuple(DESIGN_SIZES), "qwen3"), "lilalorn": (LILALORN_SIZES, "mufenex"),
+                  "debusun": (DEBUSUN_SIZES, "mufenex")}
 DESIGN_VOCAB = 32000
 MODELS = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 CONTEXT = 4096
@@ -222,18 +232,18 @@ def product(spec: str, dev="cuda:0") -> int:
 
 def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, context: int, prefill_tokens: int,
                    family: str = "both", only: str = "all") -> int:
-    """Mufenex beside Qwen3, or Lilalorn beside Mufenex, at equal sizes: ms of the prefill of one prompt and of a
-    decode step."""
+    """Mufenex beside Qwen3, or Lilalorn or Debusun beside Mufenex, at equal sizes: ms of the prefill of one prompt
+    and of a decode step."""
     import torch
     from xinfer_amd.engine import ModelRunner, StepEntry, build_model
     from xinfer_amd.models import config_from_dict
     from xinfer_amd.sampling import Sampler
     from xinfer_amd.weights.random_init import random_store_for
     name, _, size = spec.partition(":")
-    if name not in ("mufenex", "lilalorn") or (size and size not in (DESIGN_SIZES if name == "mufenex" else LILALORN_SIZES)):
-        print(f"bench.py: --design mufenex[:{'|'.join(DESIGN_SIZES)}] or lilalorn[:{'|'.join(LILALORN_SIZES)}]")
+    if name not in DESIGN_CHOICES or (size and size not in DESIGN_CHOICES[name][0]):
+        print("bench.py: --design " + " or ".join(f"{k}[:{'|'.join(v[0])}]" for k, v in DESIGN_CHOICES.items()))
         return 2
-    beside = "qwen3" if name == "mufenex" else "mufenex"
+    beside = DESIGN_CHOICES[name][1]
     if family not in ("both", name, beside):
         print(f"bench.py: --family both, {name} or {beside} with --design {name}")
         return 2
@@ -258,6 +268,24 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
                      vocab_size=DESIGN_VOCAB, sliding_window=z["window"], max_position_embeddings=2 * context)
         if name == "mufenex":
             return {"mufenex": mufenex, "qwen3": qwen3}
+        if name == "debusun":
+            # layers of a latent, windowed attention, a state space and windowed attention again, in turn; all of them
+            # are one span that runs once, so that the start of a pass is in the step
+            rot = dict(dims=z["dim"], base=500000.0)
+            lat = dict(heads=z["heads"], dim=z["dim"], vdim=z["vdim"], scale=(z["dim"] + DEBUSUN_LATENT["rot_dim"]) ** -0.5,
+                       mask={"size": z["window"]}, **DEBUSUN_LATENT,
+                       rot=dict(dims=DEBUSUN_LATENT["rot_dim"], base=500000.0,
+                                scaling=dict(factor=8.0, original=8192, fast=32.0, slow=1.0)))
+            att = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
+                       mask={"size": z["window"]}, rot=rot)
+            ssm = dict(heads=2 * z["width"] // DEBUSUN_STATE["vdim"], **DEBUSUN_STATE)
+            kinds = [("latent_attention", lat), ("attention", att), ("mamba2", ssm), ("attention", att)]
+            debusun = {"architecture": "Debusun", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+                       "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+                       "max_positions": 2 * context, "loop": {"start": 0, "stop": layers, "times": 1},
+                       "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": z["ff"]}}
+                                  for i in range(layers)]}
+            return {"debusun": debusun, "mufenex": mufenex}
         # Lilalorn: layers of attention beside retention and of gated linear attention in turn; the states' heads are a
         # quarter as many as the query heads, keys as wide as the attention's and values twice that
         mixer.pop("mask")
@@ -333,7 +361,7 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
             res.update({"prefill_ms": round(best * 1e3, 3), "prefill_tok_s": round(prefill_tokens / best, 1)})
         return res
 
-    for key in ([size] if size else list(DESIGN_SIZES if name == "mufenex" else LILALORN_SIZES)):
+    for key in ([size] if size else list(DESIGN_CHOICES[name][0])):
         z = DESIGN_SIZES[key]
         res = {k: time_model(raw) for k, raw in configs(z).items() if family in ("both", k)}
         for what in ("prefill", "decode"):
@@ -404,10 +432,10 @@ def main() -> int:
                     help="serving workloads: read every step's tokens on the host before the next step is planned")
     ap.add_argument("--product", default=None, metavar="M,N,K[,slices[,shape]]",
                     help="time one bfloat16 product alone in the many-row tiled kernel and in the vendor library")
-    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]",
-                    help="time another model family beside its closest one (Mufenex beside Qwen3, Lilalorn beside Mufenex) at equal sizes (a line of its own; --layers, --steps, "
+    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]|debusun[:SIZE]",
+                    help="time another model family beside its closest one (Mufenex beside Qwen3, Lilalorn or Debusun beside Mufenex) at equal sizes (a line of its own; --layers, --steps, "
                          "--warmup, --batch, --context, --prefill-tokens and --only apply)")
-    ap.add_argument("--family", choices=["both", "lilalorn", "mufenex", "qwen3"], default="both",
+    ap.add_argument("--family", choices=["both", "debusun", "lilalorn", "mufenex", "qwen3"], default="both",
                     help="--design: time one of the two families only (for profiling)")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "

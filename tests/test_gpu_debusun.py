@@ -210,7 +210,7 @@ LATENT_CASES = [  # H, rank, r, window, scale, L, page
 ]
 
 
-def _latent_case(case, dtype, matrix_cores, tail=9):
+def _latent_case(case, dtype, matrix_cores, tail=9, head_rows=False):
     """One pool holds [latent | turned key part] for every token, and a key's first `rank` dims are its value.  A
     sink as large as the planted scores shows in every row it belongs to; a sink of -40 must not show at all."""
     from xinfer_amd import kernels
@@ -236,6 +236,15 @@ def _latent_case(case, dtype, matrix_cores, tail=9):
             return kernels.attention_generic(qs, pool, None, table, torch.zeros_like(pos), pos, scale, window or 0, sinks=sinks,
                                              value_dim=rank)
         n, ctx = len(positions), positions[-1] + 1
+        if head_rows and n == 1:                    # the token's heads as the rows of blocks of one head
+            shape = 1 if kernels.attention_biased_block(rank + r, rank, 1, 1) >= H else 0
+            per = kernels.attention_biased_block(rank + r, rank, 1, shape)
+            tiles = _i32([[0, i * per] for i in range(-(-H // per))])
+            span = min(ctx, window + 63) if window else ctx
+            out = kernels.attention_biased_bf16(qs.view(H, 1, rank + r), pool, vt, table, tiles, _i32([0, H]), _i32([ctx]), scale,
+                                                window or 0, small=shape, split_keys=64 if positions[0] % 2 else 0, span=span,
+                                                sinks=sinks, rows_heads=H)
+            return out.view(1, H * rank)
         rows, shape = kernels.prefill_tiles([n], [ctx], rank + r, H, 1, block_of=lambda s_: kernels.attention_biased_block(rank + r, rank, H, s_))
         tiles = torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 2)
         split, span = 0, 0
@@ -262,6 +271,13 @@ def test_attention_over_a_latent_with_sinks_and_planted_keys(case, dtype):
 def test_attention_over_a_latent_on_the_matrix_cores(case):
     _latent_case(case, "bfloat16", matrix_cores=True)
     _latent_case(case, "bfloat16", matrix_cores=True, tail=70)
+
+
+@pytest.mark.parametrize("case", [c for c in LATENT_CASES if c[1] % 8 == 0 and c[2] % 8 == 0] + [(144, 136, 8, 40, 0.1, 120, 16)])
+def test_single_tokens_whose_heads_are_the_rows_of_a_block(case):
+    """Steps of single tokens over one kv head: all heads of a token in one block (or several, for many heads), whole
+    and in slices of 64 keys, each head with its own sink."""
+    _latent_case(case, "bfloat16", matrix_cores=True, tail=70, head_rows=True)
 
 
 def test_a_sink_of_the_matrix_core_kernel_with_several_kv_heads():
@@ -366,7 +382,11 @@ def test_latent_rows_and_the_heads_products(H, d, r, dv, rank, page, dtype):
     q_full = torch.zeros(L, H, rank + r, dtype=dt, device=DEV)
     kernels.latent_rows(proj_d, 0, H * (d + r), w.to(DEV), 1e-4, slots.to(DEV), pool_d, q_full, H, d, r, rank, cos, sin, True,
                         _i32(positions), values=vt_d)
-    kernels.head_linear(proj_d[:, :H * (d + r)].view(L, H, d + r)[:, :, :d], uk.to(DEV).view(H, d, rank).transpose(1, 2), q_full[:, :, :rank])
+    q_plain = proj_d[:, :H * (d + r)].view(L, H, d + r)[:, :, :d]
+    kernels.head_linear(q_plain, uk.to(DEV).view(H, d, rank).transpose(1, 2), q_full[:, :, :rank])
+    turned = torch.empty(L, H, rank, dtype=dt, device=DEV)          # U_k turned over in memory: the same product
+    kernels.head_linear(q_plain, uk.to(DEV).view(H, d, rank).transpose(1, 2).contiguous(), turned)
+    assert (turned.float() - q_full[:, :, :rank].float()).abs().max() <= (0 if dt == torch.float32 else 1e-2) * q_full.float().abs().max()
     x = proj.double()
     pos = torch.tensor(positions)
     qs = x[:, :H * (d + r)].view(L, H, d + r)
@@ -395,24 +415,28 @@ def test_latent_rows_and_the_heads_products(H, d, r, dv, rank, page, dtype):
 
 # ---- the state space ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,taps", [(40, 3), (7, 2), (130, 5), (64, 4), (9, 1)])
-def test_causal_convolution_over_portions(C, taps, dtype):
+@pytest.mark.parametrize("C,taps,pad,long", [(40, 3, 2, False), (7, 2, 2, False), (130, 5, 2, False), (64, 4, 2, False), (9, 1, 2, False),
+                                             (40, 3, 8, False), (64, 4, 8, True), (128, 5, 16, True), (16, 2, 8, True), (8, 1, 8, False),
+                                             (24, 6, 8, False)])
+def test_causal_convolution_over_portions(C, taps, pad, long, dtype):
     """Three requests in slots used before, in portions down to one token (shorter than the taps): a portion's first
-    outputs read the inputs the portion before left, a sequence's first outputs read zeros."""
+    outputs read the inputs the portion before left, a sequence's first outputs read zeros.  Channels that start at a
+    whole 16-byte chunk of rows made of such chunks take eight channels a thread, and long steps runs of tokens, with
+    sequences that start inside a run."""
     from xinfer_amd import kernels
     dt = TD[dtype]
     g = torch.Generator().manual_seed(C)
-    lens = [23, 2, 40]
-    cuts = [[2, 20, 1], [2], [1, 1, 2, 33, 3]]
+    lens = [300, 2, 1100] if long else [23, 2, 40]
+    cuts = [[2, 297, 1], [2], [1, 1, 2, 1093, 3]] if long else [[2, 20, 1], [2], [1, 1, 2, 33, 3]]
     slots = [3, 0, 2]
-    u = [(torch.randn(n, C + 3, generator=g)).to(dt) for n in lens]         # columns of wider rows
+    u = [(torch.randn(n, C + 2 * pad, generator=g)).to(dt) for n in lens]         # columns of wider rows
     wt, bias = torch.randn(C, taps, generator=g) * 0.5, torch.randn(C, generator=g) * 0.1
     tails = torch.full((5, taps - 1, C), 9.0, device=DEV)
     tails[slots] = 0                                                          # what the runner does when a request starts
     got = [[] for _ in lens]
     for rows in _steps(cuts):
         cu, tok_seq, _ = _step_index(rows)
-        x = torch.cat([u[b][a:a + n] for b, a, n in rows]).to(DEV)[:, 2:2 + C]
+        x = torch.cat([u[b][a:a + n] for b, a, n in rows]).to(DEV)[:, pad:pad + C]
         st = _i64([slots[b] for b, _, _ in rows])
         out = kernels.causal_conv(x, wt.to(DEV), bias.to(DEV), tails, st, _i32(tok_seq), _i32(cu))
         if taps > 1:
@@ -422,10 +446,12 @@ def test_causal_convolution_over_portions(C, taps, dtype):
     if taps > 1:
         assert torch.all(tails[1] == 9.0) and torch.all(tails[4] == 9.0)
     for b, n in enumerate(lens):
-        want = plain.silu(plain.causal_conv(u[b][:, 2:2 + C].double(), wt.double(), bias.double()))
-        assert (torch.cat(got[b]).double() - want).abs().max() < (1e-5 if dt == torch.float32 else 1e-2) * want.abs().max()
-        if taps > 1:
-            assert torch.equal(tails[slots[b]].cpu(), u[b][n - (taps - 1):, 2:2 + C].float()) or n < taps - 1
+        want = plain.silu(plain.causal_conv(u[b][:, pad:pad + C].double(), wt.double(), bias.double()))
+        err = (torch.cat(got[b]).double() - want).abs().max(dim=1).values
+        bad = (err > (1e-5 if dt == torch.float32 else 1e-2) * want.abs().max()).nonzero()
+        assert bad.numel() == 0, f"request {b}: first wrong token {int(bad[0])} of {n}"
+        if taps > 1 and n >= taps - 1:
+            assert torch.equal(tails[slots[b]].cpu(), u[b][n - (taps - 1):, pad:pad + C].float())
 
 
 def _ssm_inputs(T, H, G, N, dv, dt, seed):
@@ -513,18 +539,19 @@ def test_state_space_keeps_a_far_token(rate, far, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,dv,parts", [(4, 24, 2), (3, 20, 3), (2, 20, 1), (8, 64, 1), (6, 12, 6), (5, 7, 1)])
-def test_gate_before_the_norm_in_equal_parts(H, dv, parts, dtype):
+@pytest.mark.parametrize("pad", [5, 8])
+@pytest.mark.parametrize("H,dv,parts", [(4, 24, 2), (3, 20, 3), (2, 20, 1), (8, 64, 1), (6, 12, 6), (5, 7, 1), (160, 64, 1), (6, 16, 3)])
+def test_gate_before_the_norm_in_equal_parts(H, dv, parts, pad, dtype):
     from xinfer_amd import kernels
     dt = TD[dtype]
     g = torch.Generator().manual_seed(H * dv)
     T = 19
     y = torch.randn(T, H, dv, generator=g)
-    packed = torch.randn(T, 2 * H * dv + 5, generator=g).to(dt)
-    z, x = packed[:, :H * dv], packed[:, H * dv + 5:]
+    packed = torch.randn(T, 2 * H * dv + pad, generator=g).to(dt)        # z | something else | x
+    z, x = packed[:, :H * dv], packed[:, H * dv + pad:]
     skip, w = torch.randn(H, generator=g), 1 + 0.2 * torch.randn(H * dv, generator=g)
     pd = packed.to(DEV)
-    got = kernels.gated_group_norm(y.to(DEV), pd[:, H * dv + 5:], skip.to(DEV), pd[:, :H * dv], w.to(DEV), 1e-3, parts, dt)
+    got = kernels.gated_group_norm(y.to(DEV), pd[:, H * dv + pad:], skip.to(DEV), pd[:, :H * dv], w.to(DEV), 1e-3, parts, dt)
     full = y.double() + skip.double()[None, :, None] * x.double().view(T, H, dv)
     want = plain.gated_group_norm(full.reshape(T, H * dv), z.double(), w.double(), 1e-3, parts)
     assert got.dtype == dt

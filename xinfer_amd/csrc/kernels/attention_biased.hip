@@ -44,7 +44,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale,
     float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks, int window, int page_shift, int nq,
-    int nkv, int d, int dv, float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits) {
+    int nkv, int d, int dv, float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits,
+    int rows_heads) {
   const int page = 1 << page_shift;
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
@@ -67,7 +68,10 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int seq = tiles[2 * blockIdx.y], q0_blk = tiles[2 * blockIdx.y + 1];
   const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
   const int ctx = ctx_lens[seq];
-  const int pos0 = ctx - q_len;         // position of the portion's first token
+  // rows_heads > 0: the sequence's rows are the query heads of its one new token (all of them read the one kv head:
+  // attention over a latent), so every row stands at the last position and row i has sink i
+  const int step = rows_heads > 0 ? 0 : 1;
+  const int pos0 = rows_heads > 0 ? ctx - 1 : ctx - q_len;         // position of the portion's first token
   const int k_last = ctx - 1;
   {
     const int* bt = block_tables + (size_t)seq * max_pages;
@@ -77,7 +81,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
 
   // keys the workgroup walks
   const int wg_nq = min(QB, q_len - q0_blk);
-  const int wg_first = pos0 + q0_blk, wg_last = wg_first + wg_nq - 1;
+  const int wg_first = pos0 + step * q0_blk, wg_last = wg_first + step * (wg_nq - 1);
   const int wg_lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
   const int k_begin = wg_lo & ~(kKeysB - 1);
   // split_keys > 0 (steps of single tokens): this workgroup walks one slice of the keys, slice
@@ -85,6 +89,14 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int kt_begin = k_begin + (split_keys > 0 ? (int)blockIdx.z * split_keys : 0);
   const int kt_end = split_keys > 0 ? min(wg_last, kt_begin + split_keys - 1) : wg_last;
   if (split_keys > 0 && kt_begin > wg_last) {          // a slice past the sequence's keys: it says so and ends
+    if (rows_heads > 0) {                              // every row of the block (nq is 1)
+      for (int i = threadIdx.x; i < wg_nq; i += NT) {
+        float* ml = part_ml + (((size_t)(q_begin + q0_blk + i) * nq + h0) * max_splits + blockIdx.z) * 2;
+        ml[0] = -INFINITY;
+        ml[1] = 0.f;
+      }
+      return;
+    }
     for (int ct = 0; ct < NQT; ++ct) {
       const int tile = (threadIdx.x >> 6) * NQT + ct;
       if (tile < GH && (threadIdx.x & 63) == 0) {
@@ -101,7 +113,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int q0 = q0_blk + 16 * pb_lo;
   const bool active = q0 < q_len;
   const int n_q = active ? min(16 * (pb_hi - pb_lo + 1), q_len - q0) : 0;
-  const int first_pos = pos0 + q0, last_pos = first_pos + n_q - 1;
+  const int first_pos = pos0 + step * q0, last_pos = first_pos + step * (n_q - 1);
   const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
   const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
   const int wave_k_begin = lo_first & ~31;
@@ -118,7 +130,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     slope2[ct] = slopes ? slopes[h0 + hh] * kLog2eB : 0.f;
     const int qi = q0_blk + 16 * pb + r;
     const bool ok = active && qi < q_len;
-    qpos[ct] = ok ? pos0 + qi : -1;
+    qpos[ct] = ok ? pos0 + step * qi : -1;
     qlo[ct] = (ok && window > 0 && qpos[ct] - window + 1 > 0) ? qpos[ct] - window + 1 : 0;
     const bf16* qrow = q + ((size_t)(q_begin + (ok ? qi : 0)) * nq + h0 + hh) * d;
 #pragma unroll
@@ -350,7 +362,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
       continue;
     }
     // a sink: one more weight in the denominator, exp(sink) on the scale of the reference point, with no value
-    if (sinks) lt += __builtin_amdgcn_exp2f(sinks[h0 + hh] * kLog2eB - m_run[ct]);
+    if (sinks) lt += __builtin_amdgcn_exp2f(sinks[rows_heads > 0 ? qi : h0 + hh] * kLog2eB - m_run[ct]);
     const float inv = 1.f / lt;
     bf16* o = out + ((size_t)(q_begin + qi) * nq + h0 + hh) * dv;
 #pragma unroll
@@ -371,9 +383,10 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
 __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml, bf16* __restrict__ out,
                                                                  const float* __restrict__ sinks, int max_splits, int nq,
-                                                                 int dv) {
+                                                                 int dv, int rows_heads) {
   const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
-  const float sink2 = sinks ? sinks[head] * kLog2eB : -INFINITY;      // the head's sink in the exponent's unit
+  // the head's sink in the exponent's unit (rows_heads > 0: row t is head t % rows_heads of its token)
+  const float sink2 = sinks ? sinks[rows_heads > 0 ? t % rows_heads : head] * kLog2eB : -INFINITY;
   const size_t base = ((size_t)t * nq + head) * max_splits;
   __shared__ float f_s[64];
   if (max_splits <= 64) {          // a slice a lane: one round of loads for the weights, one for the sums
@@ -449,7 +462,9 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
                              int max_pages, const int* tiles, int n_tiles, const int* cu_q, const int* ctx_lens,
                              void* out, float scale, float softcap, const float* slopes, const float* sinks, int window,
                              int page, int nq, int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
-                             int max_splits, int n_tok, hipStream_t stream) {
+                             int max_splits, int n_tok, int rows_heads, hipStream_t stream) {
+  XI_CHECK(rows_heads == 0 || (rows_heads > 0 && nq == 1 && nkv == 1 && slopes == nullptr && n_tok % rows_heads == 0),
+           "attention_biased: rows that are the %d heads of a token come with one head, no slopes and whole tokens", rows_heads);
   XI_CHECK(xi_attention_biased_supported(nq, nkv, d, dv, page), "attention_biased: unsupported sizes nq=%d nkv=%d d=%d dv=%d page=%d",
            nq, nkv, d, dv, page);
   XI_CHECK(n_tiles >= 0 && n_tiles <= 65535, "attention_biased: %d query blocks are too many for one launch", n_tiles);
@@ -457,7 +472,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
   // slices of the keys: for steps in which every sequence brings one token (a tile a token), partial sums
   // part_o float32 [n_tok, nq, max_splits, dv] and part_ml [n_tok, nq, max_splits, 2] from the caller
   XI_CHECK(split_keys == 0 || (split_keys > 0 && split_keys % kKeysB == 0 && max_splits > 0 && max_splits <= 65535 &&
-                               part_o != nullptr && part_ml != nullptr && n_tiles == n_tok && dv % 4 == 0),
+                               part_o != nullptr && part_ml != nullptr && (n_tiles == n_tok || rows_heads > 0) && dv % 4 == 0),
            "attention_biased: slices of %d keys (%d of them) need steps of single tokens and room for the partial sums",
            split_keys, max_splits);
   if (n_tiles == 0) return 0;
@@ -483,7 +498,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
     kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
                                           block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
                                           scale, softcap, slopes, sinks, window, page_shift, nq, nkv, d,\
-                                          dv, part_o, part_ml, split_keys, max_splits);                 \
+                                          dv, part_o, part_ml, split_keys, max_splits, rows_heads);     \
   } while (0)
 #define XI_PB_GH(KC, DT, NQT, NWV)             \
   do {                                         \
@@ -522,7 +537,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
 #undef XI_PB
   XI_LAUNCH_CHECK("attention_biased");
   if (split_keys > 0) {
-    attn_biased_combine_kernel<<<dim3(nq, n_tok), 64, 0, stream>>>(part_o, part_ml, (bf16*)out, sinks, max_splits, nq, dv);
+    attn_biased_combine_kernel<<<dim3(nq, n_tok), 64, 0, stream>>>(part_o, part_ml, (bf16*)out, sinks, max_splits, nq, dv, rows_heads);
     XI_LAUNCH_CHECK("attention_biased_combine");
   }
   return 0;

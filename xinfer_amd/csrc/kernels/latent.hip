@@ -139,6 +139,92 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const T* __restrict__ 
   }
 }
 
+// ---- the same product on the matrix cores (bfloat16, inputs of every operand side by side) -------------------------
+// A workgroup of four waves: 128 tokens by 64 outputs of one head; wave v multiplies tokens 32 v .. 32 v + 31 by all
+// 64 outputs as 4 x 2 v_mfma_f32_16x16x32_bf16 tiles a 32-wide k step (A = 16 rows of w, B = 16 rows of x: a lane ends
+// with 4 outputs side by side of one token).  The operands go from memory straight into the lanes that multiply them,
+// a k step ahead: a wave's tokens are its own, and a head's weights are few enough to come from the caches for every
+// wave.  What lies past K is zeros; rows past the last token or output read the last one again and are dropped.  An
+// output's sum depends on K alone, never on the tokens beside it.
+typedef __attribute__((ext_vector_type(8))) __bf16 hl_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hl_f32x4;
+constexpr int kHmRows = 128, kHmCols = 64;
+
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __restrict__ x, long long x_row, long long x_head,
+                                                               const bf16* __restrict__ w, long long w_head, long long w_n,
+                                                               bf16* __restrict__ out, long long o_row, long long o_head,
+                                                               const bf16* __restrict__ gate, long long g_row,
+                                                               long long g_head, int n_tok, int N, int K) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int h = blockIdx.z;
+  const int t0 = blockIdx.x * kHmRows, n0 = blockIdx.y * kHmCols;
+  const bool wave_active = t0 + 32 * wave < n_tok;           // the same for a whole wave
+  if (!wave_active) return;
+  const bf16* xp[2];
+  const bf16* wp[4];
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    int t = t0 + 32 * wave + 16 * tj + r;
+    t = t < n_tok ? t : n_tok - 1;
+    xp[tj] = x + (size_t)h * x_head + (size_t)t * x_row + 8 * j;
+  }
+#pragma unroll
+  for (int ti = 0; ti < 4; ++ti) {
+    int n = n0 + 16 * ti + r;
+    n = n < N ? n : N - 1;
+    wp[ti] = w + (size_t)h * w_head + (size_t)n * w_n + 8 * j;
+  }
+  hl_f32x4 acc[4][2];
+#pragma unroll
+  for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) acc[ti][tj] = hl_f32x4{0.f, 0.f, 0.f, 0.f};
+  const hl_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  hl_bf16x8 a[4], b[2], an[4], bn[2];
+  const bool first = 8 * j < K;
+#pragma unroll
+  for (int ti = 0; ti < 4; ++ti) a[ti] = first ? *reinterpret_cast<const hl_bf16x8*>(wp[ti]) : zero;
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) b[tj] = first ? *reinterpret_cast<const hl_bf16x8*>(xp[tj]) : zero;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int kn = k0 + 32 + 8 * j;                           // this lane's chunk of the next step
+    const bool more = kn < K;
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti) an[ti] = more ? *reinterpret_cast<const hl_bf16x8*>(wp[ti] + k0 + 32) : zero;
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) bn[tj] = more ? *reinterpret_cast<const hl_bf16x8*>(xp[tj] + k0 + 32) : zero;
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj) acc[ti][tj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ti], b[tj], acc[ti][tj], 0, 0, 0);
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti) a[ti] = an[ti];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) b[tj] = bn[tj];
+  }
+  // a lane's 4 values of a tile: token 16 tj + r of the wave's, outputs 16 ti + 4 j .. + 3
+#pragma unroll
+  for (int tj = 0; tj < 2; ++tj) {
+    const int t = t0 + 32 * wave + 16 * tj + r;
+    if (t >= n_tok) continue;
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 16 * ti + 4 * j + i;
+        if (n >= N) continue;
+        float v = acc[ti][tj][i];
+        if (gate) {
+          const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + n]);
+          v *= 1.f / (1.f + expf(-g));
+        }
+        out[(size_t)t * o_row + (size_t)h * o_head + n] = from_float<bf16>(v);
+      }
+    }
+  }
+}
+
 }  // namespace xi
 
 using namespace xi;
@@ -184,6 +270,16 @@ int xi_head_linear(const void* x, long long x_row, long long x_head, const void*
   if (n_tok == 0) return 0;
   dim3 grid((unsigned)((n_tok + kHlRows - 1) / kHlRows), (unsigned)((N + kHlCols - 1) / kHlCols), (unsigned)H);
   XI_CHECK(grid.y <= 65535u, "head_linear: too many outputs");
+  // bfloat16 with every operand's inputs side by side in whole 16-byte chunks: the matrix cores
+  const bool chunks = K % 8 == 0 && w_k == 1 && x_row % 8 == 0 && x_head % 8 == 0 && w_head % 8 == 0 && w_n % 8 == 0 &&
+                      (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
+  if (dtype == kBF16 && chunks) {
+    dim3 mgrid((unsigned)((n_tok + kHmRows - 1) / kHmRows), (unsigned)((N + kHmCols - 1) / kHmCols), (unsigned)H);
+    head_linear_mfma_kernel<<<mgrid, 256, 0, stream>>>((const bf16*)x, x_row, x_head, (const bf16*)w, w_head, w_n, (bf16*)out,
+                                                       o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N, K);
+    XI_LAUNCH_CHECK("head_linear");
+    return 0;
+  }
   if (dtype == kF32)
     head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)w, w_head, w_n, w_k,
                                                         (float*)out, o_row, o_head, (const float*)gate, g_row, g_head, n_tok,

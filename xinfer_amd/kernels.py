@@ -1002,6 +1002,7 @@ def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first
 
 
 BIASED_MFMA = True        # False: scores with options go to the generic kernel in bfloat16 too
+HEAD_ROWS_FROM = 4        # query heads on one kv head from which a step of single tokens makes them the rows of a block
 
 
 def attention_biased_supported(nq: int, nkv: int, d: int, dv: int, page: int) -> bool:
@@ -1030,21 +1031,25 @@ def biased_split_keys(workgroups: int, span: int) -> int:
 
 
 def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, softcap=0.0,
-                          slopes=None, out=None, small=0, split_keys=0, span=0, sinks=None):
+                          slopes=None, out=None, small=0, split_keys=0, span=0, sinks=None, rows_heads=0):
     """Matrix-core attention for any mix of portions with the score's options (`softcap`, `slopes`: see
     `attention_generic`; `sinks` as there) and a value head size of its own: q [T, nq, d], K pool [pages, nkv, page, d], V pool
     [pages, nkv, page / 8, dv, 8]; tiles int32 [n, 2] = (sequence, first query token of a block of
     `attention_biased_block(d, dv, nq // nkv, small)` tokens within the sequence's portion).  Returns [T, nq * dv].
     `split_keys` > 0 (steps in which every sequence brings one token, a tile a token): each workgroup walks one slice
-    of that many keys of the up to `span` a token sees, and a second kernel puts the slices together."""
+    of that many keys of the up to `span` a token sees, and a second kernel puts the slices together.
+    `rows_heads` H > 0 (one kv head, single tokens): q is [tokens * H, 1, d], a sequence's H rows are the query heads
+    of its one new token, all at its last position, `cu_q` counts rows, `sinks` is [H] and blocks may hold many rows."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes, sinks)
     T, nq, d = q.shape
     nkv, page, dv = k_cache.shape[1], k_cache.shape[2], int(vt_cache.shape[3])
     _want(q, torch.bfloat16, "attention_biased: q")
     if sinks is not None:
         _want(sinks, torch.float32, "attention_biased: sinks")
-        if sinks.shape != (nq,):
-            raise KernelError(f"attention_biased: sinks {tuple(sinks.shape)} must be one a query head, [{nq}]")
+        if sinks.shape != (int(rows_heads) or nq,):
+            raise KernelError(f"attention_biased: sinks {tuple(sinks.shape)} must be one a query head, [{int(rows_heads) or nq}]")
+    if rows_heads and (nq != 1 or nkv != 1 or slopes is not None or T % int(rows_heads)):
+        raise KernelError("attention_biased: rows that are a token's heads come with one head, no slopes and whole tokens")
     _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv)
     for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
         _want(t, torch.int32, f"attention_biased: {name}")
@@ -1066,7 +1071,8 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
     part_o = part_ml = None
     max_splits = 0
     if split_keys:
-        if split_keys % 64 or split_keys < 0 or span <= 0 or tiles.shape[0] != T or B != T:
+        if split_keys % 64 or split_keys < 0 or span <= 0 or (not rows_heads and (tiles.shape[0] != T or B != T)) or (
+                rows_heads and B * int(rows_heads) != T):
             raise KernelError("attention_biased: slices are multiples of 64 keys, for steps of single tokens with a tile each")
         max_splits = (int(span) + 63) // int(split_keys) + 1
         part_o = torch.empty((T, nq, max_splits, dv), dtype=torch.float32, device=q.device)
@@ -1074,7 +1080,8 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
     _ok(lib().xi_attention_biased_bf16(
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
         _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), _p(sinks), int(window),
-        int(page), nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), _stream()))
+        int(page), nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), int(rows_heads),
+        _stream()))
     return out
 
 
@@ -1183,6 +1190,25 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     if softcap > 0 or slopes is not None or sinks is not None or v_cache.shape[3] != d:
         dv = int(v_cache.shape[3])
         if q.dtype == torch.bfloat16 and v_grouped and BIASED_MFMA and attention_biased_supported(nq, nkv, d, dv, page):
+            if ctx.max_q_len == 1 and nkv == 1 and nq >= HEAD_ROWS_FROM and slopes is None and q.is_contiguous():
+                # single tokens whose heads all read the one kv head: the heads are the rows of a block, so a tile
+                # of keys is read once for all of them (nothing of the step is read on the host)
+                key = ("attention_biased_head_rows", d, dv, nq)
+                cached = ctx.scratch.get(key)
+                if cached is None:
+                    small = 1 if attention_biased_block(d, dv, 1, 1) >= nq else 0
+                    rows = attention_biased_block(d, dv, 1, small)
+                    blocks = -(-nq // rows)
+                    seqs = torch.arange(ctx.num_seqs, dtype=torch.int32, device=q.device).repeat_interleave(blocks)
+                    first = (torch.arange(blocks, dtype=torch.int32, device=q.device) * rows).repeat(ctx.num_seqs)
+                    cached = (torch.stack([seqs, first], dim=1).contiguous(), small, ctx.cu_q * nq, blocks)
+                    ctx.scratch[key] = cached
+                tiles, small, cu_rows, blocks = cached
+                span = min(int(ctx.max_ctx_len), int(window) + 63) if window > 0 else int(ctx.max_ctx_len)
+                split = biased_split_keys(ctx.num_seqs * blocks, span)
+                out = attention_biased_bf16(q.view(T * nq, 1, d), k_cache, v_cache, bt, tiles, cu_rows, ctx.ctx_lens, scale, window,
+                                            softcap=softcap, small=small, split_keys=split, span=span, sinks=sinks, rows_heads=nq)
+                return out.view(T, nq * dv)
             key = ("attention_biased_tiles", d, dv, nq, nkv)
             cached = ctx.scratch.get(key)
             if cached is None:
@@ -1761,8 +1787,9 @@ def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight
 
 
 def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, h, n] = sum_k x[t, h, k] * w[h, n, k] for every head, float32 sums in ascending k; with `gate`
-    [T, H, N], out *= sigmoid(gate).  All operands may be strided views ([T, H, .] of packed rows; w [H, N, K] with
+    """out[t, h, n] = sum_k x[t, h, k] * w[h, n, k] for every head, float32 sums; with `gate`
+    [T, H, N], out *= sigmoid(gate).  bfloat16 operands whose K is contiguous in whole 16-byte chunks run on the
+    matrix cores; others, and float32, on the vector units in ascending k.  All operands may be strided views ([T, H, .] of packed rows; w [H, N, K] with
     either N or K contiguous) of one type; `out` [T, H, N] is written in place."""
     for t in (x, w, out, gate):
         if t is not None and (not t.is_cuda or t.dtype != x.dtype or t.device != x.device):

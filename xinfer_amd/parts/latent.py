@@ -64,7 +64,7 @@ class LatentAttention(Mixer):
                             and kernels.attention_biased_supported(self.heads, 1, self.rank + self.r, self.rank, 64))
         self.proj: Optional[Linear] = None          # [q | dkv | g] rows
         self.o: Optional[Linear] = None
-        self.uk = self.uv = None                    # [heads, dim, rank] and [heads, vdim, rank], as stored
+        self.uk = self.uv = None                    # [heads, rank, dim] (turned over) and [heads, vdim, rank] (as stored)
         self.norm_w = self.sinks = None
 
     @classmethod
@@ -93,7 +93,8 @@ class LatentAttention(Mixer):
         parts = [self._lin(store, n[k], device) for k in (("q", "dkv", "g") if self.has_gate else ("q", "dkv"))]
         self.proj = Linear(torch.cat([p.to(self.dtype) for p in parts], dim=0))
         self.o = Linear(self._lin(store, n["o"], device).to(self.dtype))
-        self.uk = self._lin(store, n["uk"], device).to(self.dtype).contiguous().view(self.heads, self.d, self.rank)
+        # U_k with a head's inputs (its plain query dims) side by side, as the queries' product reads it
+        self.uk = self._lin(store, n["uk"], device).to(self.dtype).view(self.heads, self.d, self.rank).transpose(1, 2).contiguous()
         self.uv = self._lin(store, n["uv"], device).to(self.dtype).contiguous().view(self.heads, self.dv, self.rank)
         self.norm_w = store.get(n["dkv_norm"], torch.float32, device).contiguous()
         if self.has_sinks:
@@ -122,7 +123,7 @@ class LatentAttention(Mixer):
                             pos.interleaved, ctx.positions, values=values)
         # the plain part of every head's query through its U_k: out[t, h, j] = sum_i q[t, h, i] U_k[h, i, j]
         q_plain = p[:, :q_cols].view(T, H, d + r)[:, :, :d]
-        kernels.head_linear(q_plain, self.uk.transpose(1, 2), q_full[:, :, :rank])
+        kernels.head_linear(q_plain, self.uk, q_full[:, :, :rank])
         a = kernels.attention(q_full, pool, values, ctx, cache.group, self.scale, self.window, v_grouped=values is not None,
                               sinks=self.sinks, value_dim=rank)
         # the heads' weighted sums of the latent through their U_v, times the gate
