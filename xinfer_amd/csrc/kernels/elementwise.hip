@@ -798,6 +798,31 @@ __global__ void act_kernel(T* __restrict__ x, size_t n) {
   x[i] = from_float<T>(r);
 }
 
+// The same for bfloat16 in whole 16-byte chunks: eight elements a thread.
+template <int ACT>
+__global__ void act_vec8_kernel(bf16* __restrict__ x, size_t chunks) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= chunks) return;
+  uint4* p = reinterpret_cast<uint4*>(x) + i;
+  const uint4 a = *p;
+  unsigned u[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float z[2] = {__uint_as_float(u[k] << 16), __uint_as_float(u[k] & 0xffff0000u)};
+    unsigned short o[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      float r;
+      if constexpr (ACT == 2) r = z[e] > 0.f ? z[e] * z[e] : 0.f;
+      else r = act_of<ACT>(z[e]);
+      const bf16 b = __float2bfloat16(r);
+      o[e] = *reinterpret_cast<const unsigned short*>(&b);
+    }
+    u[k] = (unsigned)o[0] | ((unsigned)o[1] << 16);
+  }
+  *p = make_uint4(u[0], u[1], u[2], u[3]);
+}
+
 // out[t, :] += sigmoid(gate[t * gate_stride]) * y[t, :]   (out float32; one number a token opens the branch)
 template <typename T>
 __global__ void gated_add_kernel(float* __restrict__ out, const T* __restrict__ y, const float* __restrict__ gate,
@@ -833,6 +858,15 @@ int xi_scale(float* x, int64_t n, float factor, hipStream_t stream) {
 int xi_act(void* x, int dtype, int act, int64_t n, hipStream_t stream) {
   XI_CHECK(n >= 0 && act >= 0 && act <= 2, "act: bad size or unknown activation %d", act);
   if (n == 0) return 0;
+  if (dtype == kBF16 && n % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const size_t chunks = (size_t)n / 8;
+    const unsigned vblocks = (unsigned)((chunks + 255) / 256);
+    if (act == 0) act_vec8_kernel<0><<<vblocks, 256, 0, stream>>>((bf16*)x, chunks);
+    else if (act == 1) act_vec8_kernel<1><<<vblocks, 256, 0, stream>>>((bf16*)x, chunks);
+    else act_vec8_kernel<2><<<vblocks, 256, 0, stream>>>((bf16*)x, chunks);
+    XI_LAUNCH_CHECK("act");
+    return 0;
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256);
 #define XI_ACT(TT)                                                                  \
   do {                                                                              \

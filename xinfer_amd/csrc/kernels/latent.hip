@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
                                                                const bf16* __restrict__ w, long long w_head, long long w_n,
                                                                bf16* __restrict__ out, long long o_row, long long o_head,
                                                                const bf16* __restrict__ gate, long long g_row,
-                                                               long long g_head, int n_tok, int N, int K) {
+                                                               long long g_head, int n_tok, int N, int K, int wide) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int h = blockIdx.z;
@@ -210,9 +210,29 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
     if (t >= n_tok) continue;
 #pragma unroll
     for (int ti = 0; ti < 4; ++ti) {
+      const int nf = n0 + 16 * ti + 4 * j;
+      if (wide && nf + 3 < N) {              // the lane's 4 outputs in one 8-byte store (and one load of the gate)
+        float v[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
+        if (gate) {
+          const uint2 gb = *reinterpret_cast<const uint2*>(gate + (size_t)t * g_row + (size_t)h * g_head + nf);
+          const float g4[4] = {__uint_as_float(gb.x << 16), __uint_as_float(gb.x & 0xffff0000u), __uint_as_float(gb.y << 16),
+                               __uint_as_float(gb.y & 0xffff0000u)};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= 1.f / (1.f + expf(-g4[i]));
+        }
+        unsigned short b4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bf16 o = __float2bfloat16(v[i]);
+          b4[i] = *reinterpret_cast<const unsigned short*>(&o);
+        }
+        *reinterpret_cast<uint2*>(out + (size_t)t * o_row + (size_t)h * o_head + nf) =
+            make_uint2((unsigned)b4[0] | ((unsigned)b4[1] << 16), (unsigned)b4[2] | ((unsigned)b4[3] << 16));
+        continue;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 16 * ti + 4 * j + i;
+        const int n = nf + i;
         if (n >= N) continue;
         float v = acc[ti][tj][i];
         if (gate) {
@@ -275,8 +295,11 @@ int xi_head_linear(const void* x, long long x_row, long long x_head, const void*
                       (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0;
   if (dtype == kBF16 && chunks) {
     dim3 mgrid((unsigned)((n_tok + kHmRows - 1) / kHmRows), (unsigned)((N + kHmCols - 1) / kHmCols), (unsigned)H);
+    // outputs (and the gate) in 8-byte pieces where every lane's 4 outputs start at one
+    const int wide = o_row % 4 == 0 && o_head % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 &&
+                     (gate == nullptr || (g_row % 4 == 0 && g_head % 4 == 0 && (reinterpret_cast<uintptr_t>(gate) & 7) == 0));
     head_linear_mfma_kernel<<<mgrid, 256, 0, stream>>>((const bf16*)x, x_row, x_head, (const bf16*)w, w_head, w_n, (bf16*)out,
-                                                       o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N, K);
+                                                       o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N, K, wide);
     XI_LAUNCH_CHECK("head_linear");
     return 0;
   }
