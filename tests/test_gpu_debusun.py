@@ -579,7 +579,7 @@ def test_the_start_of_a_pass(width):
 
 # ---- whole models ----------------------------------------------------------------------------------------------------
 LENGTHS = {"A": [1, 2, 12, 13, 33, 77, 130], "B": [3, 9, 10, 18, 64, 101], "C": [1, 7, 8, 40, 75, 210], "D": [2, 1, 30, 140],
-           "R": [5, 101, 330, 64, 301]}
+           "R": [5, 101, 330, 64, 301], "S": [3, 70, 71, 260, 129]}
 
 
 def _requests(name):
@@ -703,7 +703,7 @@ def test_short_chunks_of_the_states_walk(name, dtype, dirs, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "R"])
+@pytest.mark.parametrize("name", ["A", "B", "R", "S"])
 def test_unequal_requests_decoding_together(name, dtype, dirs):
     reqs = {k: v for k, v in _requests(name).items() if len(v) > 8}
     reqs = dict(list(reqs.items())[:4])
