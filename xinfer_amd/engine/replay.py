@@ -62,8 +62,8 @@ def main(argv=None) -> int:
                 next_id += 1
                 runner.add_request(ids[key])
             entries.append(StepEntry(ids[key], e["tokens"], e.get("want", [])))
-        logits = runner.step(entries)
-        if logits.shape[0] > 0:
+        logits = runner.step(entries) if entries else None      # a step may only end requests
+        if logits is not None and logits.shape[0] > 0:
             arr = logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4", copy=False)
             tmp = os.path.join(args.out, f".{step}.f32.tmp")
             arr.tofile(tmp)
