@@ -13,7 +13,8 @@ D: a span that runs once (its table has one row); a latent layer last; a window 
 R: real-looking head sizes (64 and 128, a latent of 128 + 32) with pages of 64, for the matrix-core kernels.
 S: the matrix-core kernels' sizes again with what R leaves out: equal key and value head sizes of which only a part
    turns (half of 64, a quarter of 128), a latent of 64 + 16 for 6 heads with values wider than the plain key dims, a
-   state space with 3 groups and states of 32; the span is the first two layers, three times.
+   state space with 3 groups and states of 32; the span is the state space and the latent, twice (a latent on the
+   matrix cores with a cache a pass).
 """
 import os
 
@@ -86,7 +87,7 @@ MODELS = {
         _att(4, 2, 64, 64, 0.125, 70, _rot(32, 10000.0), 256),
         _att(2, 1, 128, 128, 0.09, 200, _rot(32, 500000.0), None),
         _ssm(6, 32, 32, 3, 4, 2, 320),
-        _lat(6, 32, 16, 48, 64, 0.14, 90, _rot(16, 10000.0, (4.0, 128, 16.0, 2.0)), 256)], loop=(0, 2, 3)),
+        _lat(6, 32, 16, 48, 64, 0.14, 90, _rot(16, 10000.0, (4.0, 128, 16.0, 2.0)), 256)], loop=(2, 4, 2)),
         seed=26, linear_std=0.05, norm_std=0.1, page_size=64),
 }
 
