@@ -49,7 +49,9 @@ __device__ __forceinline__ float decay_of(float z, float inv_tau) {
   return expf(-sp * inv_tau);
 }
 
-template <typename T, int RPT>
+// ONE: a token's decay is one number for all of a head's channels (a constant per head, or from a step size): every
+// thread makes it itself and keeps it in a register, and the decays' row in LDS is neither written nor read.
+template <typename T, int RPT, bool ONE>
 __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
     long long v_stride, const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau,
@@ -90,8 +92,9 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     if (c < dk) {
       fq = to_float(q[(size_t)t * q_stride + qk0 + c]) * q_scale;
       fk = to_float(k[(size_t)t * k_stride + qk0 + c]) * k_scale;
-      fa = step ? expf(rate * dt) : z ? decay_of(z[((size_t)t * H + h) * dk + c] + zb, inv_tau) : hd;
+      if (!ONE) fa = decay_of(z[((size_t)t * H + h) * dk + c] + zb, inv_tau);
     }
+    if (ONE) fa = step ? expf(rate * dt) : hd;
   };
   float fq = 0.f, fk = 0.f, fa = 0.f;
   float dt = step_of(t0);
@@ -100,11 +103,12 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   float v_next = col ? to_float(v[(size_t)t0 * v_stride + h * dv + j]) * dt : 0.f;
   qs[0][c] = fq;
   ks[0][c] = fk;
-  as[0][c] = fa;
+  if (!ONE) as[0][c] = fa;
   __syncthreads();
   for (int t = t0; t < t1; ++t) {
     const int cur = (t - t0) & 1;
     all_decays *= fa;
+    const float a_now = fa;
     const float vj = v_next;
     if (t + 1 < t1) {
       dt = step_of(t + 1);
@@ -117,7 +121,8 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     const float4* q4 = reinterpret_cast<const float4*>(&qs[cur][wave * RPT]);
 #pragma unroll
     for (int r = 0; r < RPT; r += 4) {
-      const float4 av = a4[r / 4], kv = k4[r / 4], qv = q4[r / 4];
+      const float4 av = ONE ? make_float4(a_now, a_now, a_now, a_now) : a4[r / 4];
+      const float4 kv = k4[r / 4], qv = q4[r / 4];
       s[r] = fmaf(av.x, s[r], kv.x * vj);
       s[r + 1] = fmaf(av.y, s[r + 1], kv.y * vj);
       s[r + 2] = fmaf(av.z, s[r + 2], kv.z * vj);
@@ -131,7 +136,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     if (t + 1 < t1) {
       qs[cur ^ 1][c] = fq;
       ks[cur ^ 1][c] = fk;
-      as[cur ^ 1][c] = fa;
+      if (!ONE) as[cur ^ 1][c] = fa;
     }
     __syncthreads();
     if (out && wave == 0 && col)
@@ -230,11 +235,15 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
   XI_CHECK(grid.y <= 65535u && grid.z <= 65535u, "linear_scan: too many heads or value columns");
   const float inv_tau = z ? 1.f / tau : 0.f;
   const int rpt = (dk + kScanWaves - 1) / kScanWaves;
-#define XI_SCAN(TT, R)                                                                                                        \
-  linear_scan_kernel<TT, R><<<grid, kScanWaves * kWave, 0, stream>>>(                                                         \
+#define XI_SCAN_ARGS(TT)                                                                                                      \
       (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, (const TT*)step,    \
       step_stride, step_bias, decay_log, group_heads, state_in, in_stride,                                                    \
-      in_idx, state_out, out_stride, out_idx, first, last, out, decay_out, H, dk, dv, q_scale, k_scale)
+      in_idx, state_out, out_stride, out_idx, first, last, out, decay_out, H, dk, dv, q_scale, k_scale
+#define XI_SCAN(TT, R)                                                                                                        \
+  do {                                                                                                                        \
+    if (z) linear_scan_kernel<TT, R, false><<<grid, kScanWaves * kWave, 0, stream>>>(XI_SCAN_ARGS(TT));                       \
+    else linear_scan_kernel<TT, R, true><<<grid, kScanWaves * kWave, 0, stream>>>(XI_SCAN_ARGS(TT));                          \
+  } while (0)
 #define XI_SCAN_T(TT)            \
   do {                           \
     if (rpt <= 8) XI_SCAN(TT, 8); \
@@ -247,6 +256,7 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
   else XI_CHECK(false, "linear_scan: unknown dtype %d", dtype);
 #undef XI_SCAN_T
 #undef XI_SCAN
+#undef XI_SCAN_ARGS
   XI_LAUNCH_CHECK("linear_scan");
   return 0;
 }
