@@ -464,7 +464,8 @@ def _ssm_inputs(T, H, G, N, dv, dt, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chunk", [0, 16])
-@pytest.mark.parametrize("H,G,N,dv", [(4, 2, 16, 24), (3, 3, 8, 20), (2, 1, 12, 20), (8, 1, 64, 64), (6, 3, 16, 12), (1, 1, 128, 8)])
+@pytest.mark.parametrize("H,G,N,dv", [(4, 2, 16, 24), (3, 3, 8, 20), (2, 1, 12, 20), (8, 1, 64, 64), (6, 3, 16, 12), (1, 1, 128, 8),
+                                      (2, 1, 40, 80), (4, 2, 256, 136)])
 def test_state_space_walk_of_unequal_requests_in_portions(H, G, N, dv, chunk, dtype, monkeypatch):
     from xinfer_amd import kernels
     monkeypatch.setattr(kernels, "SCAN_CHUNK", chunk)
