@@ -9,6 +9,8 @@
 //     and key position j; then the mask (causal, window).  tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1):
 //     one exponential and one reciprocal a score beside the softmax's own exponential, which is
 //     why this kernel spends more of its time outside the matrix cores than the plain one.
+//   - a K pool of fewer heads than the V pool (`nkk`, a divisor of nkv: kv head c reads key head c / (nkv / nkk));
+//     one key head of all kv heads' dims side by side serves heads whose scores are mixed.
 // It serves every mix of prompt portions and single tokens (a single token is a block of one
 // query position); the host lays out `tiles` as for the plain kernel.
 #include "common.h"
@@ -45,7 +47,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale,
     float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks, int window, int page_shift, int nq,
     int nkv, int d, int dv, float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits,
-    int rows_heads) {
+    int rows_heads, int nkk) {
   const int page = 1 << page_shift;
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
@@ -65,6 +67,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int g = nq / nkv, groups = g / GH;
   const int kvh = blockIdx.x / groups;
   const int h0 = kvh * g + (blockIdx.x - kvh * groups) * GH;
+  const int kh = kvh / (nkv / nkk);               // the kv head's key head
   const int seq = tiles[2 * blockIdx.y], q0_blk = tiles[2 * blockIdx.y + 1];
   const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
   const int ctx = ctx_lens[seq];
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
       int key = kb + c_kl[i];
       key = key > k_last ? k_last : key;
       const int kp = bt_s[key >> page_shift];
-      const bf16* ksrc = k_cache + ((size_t)kp * nkv + kvh) * k_head_stride +
+      const bf16* ksrc = k_cache + ((size_t)kp * nkk + kh) * k_head_stride +
                          (size_t)(key & (page - 1)) * d + (c_koff[i] < 0 ? 0 : c_koff[i]);
       kreg[i] = ld8(ksrc);
     }
@@ -462,7 +465,8 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
                              int max_pages, const int* tiles, int n_tiles, const int* cu_q, const int* ctx_lens,
                              void* out, float scale, float softcap, const float* slopes, const float* sinks, int window,
                              int page, int nq, int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
-                             int max_splits, int n_tok, int rows_heads, hipStream_t stream) {
+                             int max_splits, int n_tok, int rows_heads, int nkk, hipStream_t stream) {
+  XI_CHECK(nkk > 0 && nkv % nkk == 0, "attention_biased: %d kv heads on %d key heads", nkv, nkk);
   XI_CHECK(rows_heads == 0 || (rows_heads > 0 && nq == 1 && nkv == 1 && slopes == nullptr && n_tok % rows_heads == 0),
            "attention_biased: rows that are the %d heads of a token come with one head, no slopes and whole tokens", rows_heads);
   XI_CHECK(xi_attention_biased_supported(nq, nkv, d, dv, page), "attention_biased: unsupported sizes nq=%d nkv=%d d=%d dv=%d page=%d",
@@ -498,7 +502,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
     kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
                                           block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
                                           scale, softcap, slopes, sinks, window, page_shift, nq, nkv, d,\
-                                          dv, part_o, part_ml, split_keys, max_splits, rows_heads);     \
+                                          dv, part_o, part_ml, split_keys, max_splits, rows_heads, nkk);\
   } while (0)
 #define XI_PB_GH(KC, DT, NQT, NWV)             \
   do {                                         \

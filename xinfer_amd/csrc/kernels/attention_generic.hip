@@ -11,6 +11,8 @@
 // with the distance to the key).  With per-head `sinks` z[h] the softmax's denominator also holds
 // exp(z[h]): one more weight, taken as it is, that no value goes with.  With `values_in_keys`
 // there is no V pool: a key's first dv dims are its value (attention over a latent).
+// The K pool may hold another number of heads than the V pool, `nkk` (query head h reads key head h / (nq / nkk) and
+// value head h / (nq / nkv)): one key head of all kv heads' dims side by side serves heads whose scores are mixed.
 //
 // Reference: PagedAttention::forward at /root/reference/src/models/layers/attention.rs:947-958
 // (external kernel); golden formula tests/probes/compare_flashinfer_probe.py:51-73:
@@ -34,7 +36,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, T* __restrict__ out, float scale, int window, int page_size,
     int nq, int nkv, int d, int dv, int v_grouped, float softcap, const float* __restrict__ slopes,
-    const float* __restrict__ sinks, int values_in_keys) {
+    const float* __restrict__ sinks, int values_in_keys, int nkk) {
   __shared__ float q_s[MAXD];
   __shared__ float acc_s[kAttnWaves][MAXD];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
@@ -42,6 +44,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
   const int t = blockIdx.x;
   const int h = blockIdx.y;
   const int kvh = h / (nq / nkv);
+  const int kh = h / (nq / nkk);
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int seq = tok_seq[t];
@@ -67,11 +70,13 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const int key = lo + c * kWave + lane;
     const bool valid = key <= pos;
     int row = 0;  // row of this lane's key in the cache, in units of d elements
+    int val = 0;  // and of its value, in units of dv elements
     int vrow = 0, voff = 0;  // grouped V: first row of the (page, kv head) block and the offset
     float s = -INFINITY;
     if (valid) {
       const int page = bt[key / page_size];
-      row = (page * nkv + kvh) * page_size + key % page_size;
+      row = (page * nkk + kh) * page_size + key % page_size;
+      val = (page * nkv + kvh) * page_size + key % page_size;
       vrow = (page * nkv + kvh) * dv;
       voff = key % page_size;
       const T* kp = k_cache + (size_t)row * d;
@@ -91,7 +96,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const int n_in_chunk = min(kWave, pos - (lo + c * kWave) + 1);
     for (int j = 0; j < n_in_chunk; ++j) {
       const float pj = __shfl(p, j, kWave);
-      const int rj = __shfl(row, j, kWave);
+      const int rj = __shfl(values_in_keys ? row : val, j, kWave);
       const int vrj = __shfl(vrow, j, kWave);
       const int voj = __shfl(voff, j, kWave);
       const T* vp = values_in_keys ? k_cache + (size_t)rj * d : v_cache + (size_t)rj * dv;
@@ -147,10 +152,11 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
                                     const int* tok_seq, const int* positions, void* out,
                                     float scale, int window, int page_size, int n_tok, int nq,
                                     int nkv, int d, int dv, int v_grouped, float softcap, const float* slopes,
-                                    const float* sinks, int values_in_keys, hipStream_t stream) {
+                                    const float* sinks, int values_in_keys, int nkk, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && page_size > 0 && max_pages > 0,
            "attention: bad sizes T=%d nq=%d nkv=%d page=%d max_pages=%d", n_tok, nq, nkv, page_size, max_pages);
   XI_CHECK(nq % nkv == 0, "attention: %d query heads are not a multiple of %d kv heads", nq, nkv);
+  XI_CHECK(nkk > 0 && nq % nkk == 0 && (!values_in_keys || nkk == nkv), "attention: %d query heads on %d key heads", nq, nkk);
   XI_CHECK(d > 0 && d <= kMaxHeadDimWide, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDimWide);
   XI_CHECK(dv > 0 && dv <= kMaxHeadDimWide, "attention: value head size %d is outside 1..%d", dv, kMaxHeadDimWide);
   XI_CHECK(!values_in_keys || (dv <= d && !v_grouped), "attention: values that are the keys' first dims need dv <= d");
@@ -163,7 +169,7 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
 #define XI_AG(TT, MAXD)                                                                                                 \
   attention_generic_kernel<TT, MAXD><<<grid, kAttnWaves * kWave, 0, stream>>>(                                          \
       (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, block_tables, max_pages, tok_seq, positions, (TT*)out, scale, \
-      window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes, sinks, values_in_keys)
+      window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes, sinks, values_in_keys, nkk)
   if (dtype == kF32 && !wide) XI_AG(float, kMaxHeadDim);
   else if (dtype == kF32) XI_AG(float, kMaxHeadDimWide);
   else if (dtype == kBF16 && !wide) XI_AG(bf16, kMaxHeadDim);

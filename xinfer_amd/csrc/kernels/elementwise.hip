@@ -585,6 +585,8 @@ __global__ __launch_bounds__(NT) void rmsnorm_add_vec_kernel(float* __restrict__
 // ---------------------------------------------------------------------------------
 // act(gate) * up for a packed [T, 2I] buffer, the activation chosen by code:
 // 0 silu(z) = z * sigmoid(z); 1 the tanh form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// With `row_scale` s (float32, row t's factor at s[row_of ? row_of[t] : t]) gate and up are multiplied by it
+// first: what a factor on the INPUT of the two (linear) products makes of them.
 // ---------------------------------------------------------------------------------
 enum Act : int { kSilu = 0, kGeluTanh = 1 };
 template <int ACT>
@@ -593,24 +595,28 @@ __device__ __forceinline__ float act_of(float z) {
   else return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 template <typename T, int ACT>
-__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total,
+                               const float* __restrict__ row_scale, const int* __restrict__ row_of) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / I, i = idx - t * I;
-    const float g = to_float(gu[t * 2 * I + i]), u = to_float(gu[t * 2 * I + I + i]);
+    const float sc = row_scale ? row_scale[row_of ? row_of[t] : t] : 1.f;
+    const float g = to_float(gu[t * 2 * I + i]) * sc, u = to_float(gu[t * 2 * I + I + i]) * sc;
     out[idx] = from_float<T>(act_of<ACT>(g) * u);
   }
 }
 
 template <int ACT>
-__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int I, size_t total8) {
+__global__ void act_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int I, size_t total8,
+                                    const float* __restrict__ row_scale, const int* __restrict__ row_of) {
   const int I8 = I / 8;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / I8, i = (idx - t * I8) * 8;
+    const float sc = row_scale ? row_scale[row_of ? row_of[t] : t] : 1.f;
     const bf16x8_t g = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + i);
     const bf16x8_t u = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + I + i);
     bf16x8_t o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16>(act_of<ACT>(to_float(g.v[e])) * to_float(u.v[e]));
+    for (int e = 0; e < 8; ++e) o.v[e] = from_float<bf16>(act_of<ACT>(to_float(g.v[e]) * sc) * (to_float(u.v[e]) * sc));
     *reinterpret_cast<bf16x8_t*>(out + t * I + i) = o;
   }
 }
@@ -1103,20 +1109,24 @@ int xi_rmsnorm_add(float* resid, const void* y, int y_dtype, int parts, const fl
   return 0;
 }
 
-int xi_act_mul(const void* gate_up, void* out, int dtype, int act, int n_tok, int I, hipStream_t stream) {
+int xi_act_mul(const void* gate_up, void* out, int dtype, int act, int n_tok, int I, const float* row_scale, const int* row_of,
+               hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && I > 0, "act_mul: bad sizes T=%d I=%d", n_tok, I);
   XI_CHECK(act == kSilu || act == kGeluTanh, "act_mul: unknown activation %d", act);
   if (n_tok == 0) return 0;
   const size_t total = (size_t)n_tok * I;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
-#define XI_AM(TT, A) act_mul_kernel<TT, A><<<(unsigned)blocks, 256, 0, stream>>>((const TT*)gate_up, (TT*)out, I, total)
+#define XI_AM(TT, A) \
+  act_mul_kernel<TT, A><<<(unsigned)blocks, 256, 0, stream>>>((const TT*)gate_up, (TT*)out, I, total, row_scale, row_of)
   if (dtype == kBF16 && I % 8 == 0 && ((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0) {
     const size_t total8 = total / 8;
     size_t b8 = (total8 + 255) / 256;
     if (b8 > 65535u * 16u) b8 = 65535u * 16u;
-    if (act == kSilu) act_mul_vec8_kernel<kSilu><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8);
-    else act_mul_vec8_kernel<kGeluTanh><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8);
+    if (act == kSilu)
+      act_mul_vec8_kernel<kSilu><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8, row_scale, row_of);
+    else
+      act_mul_vec8_kernel<kGeluTanh><<<(unsigned)b8, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8, row_scale, row_of);
   } else if (dtype == kF32 && act == kSilu) XI_AM(float, kSilu);
   else if (dtype == kF32) XI_AM(float, kGeluTanh);
   else if (dtype == kBF16 && act == kSilu) XI_AM(bf16, kSilu);

@@ -10,7 +10,7 @@
 //
 // `latent_rows_kernel`, a workgroup a token, from the packed projection row [q (H (dim + r)) | down (rank + r) | ..]:
 //   c = down[:rank] / sqrt(mean(down[:rank]^2) + eps) * w   and the turned down[rank:] into the pool at the slot;
-//   every head's turned q part into q_full[t, h, rank:].
+//   every head's turned q part into q_full[t, h, rank:] (the q parts may be rows of another tensor, `q_rows`).
 // Pairs (2i, 2i + 1) or (i, i + r / 2) turn by the position's row of float32 tables [positions, r / 2].
 //
 // `head_linear_kernel`: out[t, h, n] = sum_k x[t, h, k] * w[h][n][k] for every head, with the strides of all
@@ -27,10 +27,12 @@ __global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ 
                                                           T* __restrict__ values, int page_size, T* __restrict__ q_full, int H, int dim, int r,
                                                           int rank, const float* __restrict__ cos_t,
                                                           const float* __restrict__ sin_t, int interleaved,
-                                                          const int* __restrict__ positions) {
+                                                          const int* __restrict__ positions, const T* __restrict__ q_rows,
+                                                          long long q_stride) {
   __shared__ float scratch[4];
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * proj_stride;
+  const T* qrow = q_rows + (size_t)t * q_stride;       // the heads' q parts: the same rows, or rows of their own
   const int half = r / 2;
   const size_t trow = (size_t)positions[t] * half;
   // the heads' turned parts
@@ -38,7 +40,7 @@ __global__ __launch_bounds__(256) void latent_rows_kernel(const T* __restrict__ 
   for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
     const int h = i / half, p = i - h * half;
     const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : p + half;
-    const T* src = row + q_off + (size_t)h * (dim + r) + dim;
+    const T* src = qrow + q_off + (size_t)h * (dim + r) + dim;
     const float a = to_float(src[ia]), b = to_float(src[ib]);
     const float cs = cos_t[trow + p], sn = sin_t[trow + p];
     T* dst = qf + (size_t)h * (rank + r) + rank;
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const T* __restrict__ 
                                                           const T* __restrict__ w, long long w_head, long long w_n,
                                                           long long w_k, T* __restrict__ out, long long o_row,
                                                           long long o_head, const T* __restrict__ gate, long long g_row,
-                                                          long long g_head, int n_tok, int N, int K) {
+                                                          long long g_head, int g_each, int n_tok, int N, int K) {
   __shared__ float xs[kHlK][kHlRows + 1];
   __shared__ float ws[kHlK][kHlCols + 1];
   const int h = blockIdx.z;
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const T* __restrict__ 
       if (n >= N) continue;
       float v = acc[i][j];
       if (gate) {
-        const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + n]);
+        const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + (g_each ? n : 0)]);
         v *= 1.f / (1.f + expf(-g));
       }
       out[(size_t)t * o_row + (size_t)h * o_head + n] = from_float<T>(v);
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
                                                                const bf16* __restrict__ w, long long w_head, long long w_n,
                                                                bf16* __restrict__ out, long long o_row, long long o_head,
                                                                const bf16* __restrict__ gate, long long g_row,
-                                                               long long g_head, int n_tok, int N, int K, int wide) {
+                                                               long long g_head, int g_each, int n_tok, int N, int K, int wide) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int h = blockIdx.z;
@@ -213,7 +215,11 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
       const int nf = n0 + 16 * ti + 4 * j;
       if (wide && nf + 3 < N) {              // the lane's 4 outputs in one 8-byte store (and one load of the gate)
         float v[4] = {acc[ti][tj][0], acc[ti][tj][1], acc[ti][tj][2], acc[ti][tj][3]};
-        if (gate) {
+        if (gate && !g_each) {                   // one number a head
+          const float sg = 1.f / (1.f + expf(-to_float(gate[(size_t)t * g_row + (size_t)h * g_head])));
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= sg;
+        } else if (gate) {
           const uint2 gb = *reinterpret_cast<const uint2*>(gate + (size_t)t * g_row + (size_t)h * g_head + nf);
           const float g4[4] = {__uint_as_float(gb.x << 16), __uint_as_float(gb.x & 0xffff0000u), __uint_as_float(gb.y << 16),
                                __uint_as_float(gb.y & 0xffff0000u)};
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16* __res
         if (n >= N) continue;
         float v = acc[ti][tj][i];
         if (gate) {
-          const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + n]);
+          const float g = to_float(gate[(size_t)t * g_row + (size_t)h * g_head + (g_each ? n : 0)]);
           v *= 1.f / (1.f + expf(-g));
         }
         out[(size_t)t * o_row + (size_t)h * o_head + n] = from_float<bf16>(v);
@@ -255,10 +261,15 @@ extern "C" {
 // down_off; w float32 [rank]; pool [pages, 1, page, rank + r]; q_full [T, H, rank + r] (its last r dims are written).
 int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_off, int dtype, const float* w, float eps,
                    const long long* slots, void* pool, void* values, int page_size, void* q_full, int n_tok, int H, int dim, int r, int rank,
-                   const float* cos_t, const float* sin_t, int interleaved, const int* positions, hipStream_t stream) {
+                   const float* cos_t, const float* sin_t, int interleaved, const int* positions, const void* q_rows,
+                   long long q_stride, hipStream_t stream) {
+  if (q_rows == nullptr) {
+    q_rows = proj;
+    q_stride = proj_stride;
+  }
   XI_CHECK(n_tok >= 0 && H > 0 && dim > 0 && r >= 0 && r % 2 == 0 && rank > 0 && page_size > 0,
            "latent_rows: bad sizes T=%d H=%d dim=%d r=%d rank=%d page=%d", n_tok, H, dim, r, rank, page_size);
-  XI_CHECK(q_off >= 0 && down_off >= 0 && proj_stride >= (long long)q_off + (long long)H * (dim + r) &&
+  XI_CHECK(q_off >= 0 && down_off >= 0 && q_stride >= (long long)q_off + (long long)H * (dim + r) &&
                proj_stride >= (long long)down_off + rank + r,
            "latent_rows: the projection's rows are too short");
   XI_CHECK(r == 0 || (cos_t && sin_t), "latent_rows: a rotation needs its tables");
@@ -268,11 +279,11 @@ int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_
   if (dtype == kF32)
     latent_rows_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)proj, proj_stride, q_off, down_off, w, eps, slots,
                                                          (float*)pool, (float*)values, page_size, (float*)q_full, H, dim, r, rank, cos_t,
-                                                         sin_t, interleaved, positions);
+                                                         sin_t, interleaved, positions, (const float*)q_rows, q_stride);
   else if (dtype == kBF16)
     latent_rows_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)proj, proj_stride, q_off, down_off, w, eps, slots,
                                                         (bf16*)pool, (bf16*)values, page_size, (bf16*)q_full, H, dim, r, rank, cos_t, sin_t,
-                                                        interleaved, positions);
+                                                        interleaved, positions, (const bf16*)q_rows, q_stride);
   else
     XI_CHECK(false, "latent_rows: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("latent_rows");
@@ -280,10 +291,11 @@ int xi_latent_rows(const void* proj, long long proj_stride, int q_off, int down_
 }
 
 // x: token t, head h, element k at x + t x_row + h x_head + k; w: head h, output n, element k at w + h w_head + n w_n +
-// k w_k (one of w_n, w_k is 1); out: at out + t o_row + h o_head + n; gate null or laid out like out with its own strides.
+// k w_k (one of w_n, w_k is 1); out: at out + t o_row + h o_head + n; gate null or laid out like out with its own strides,
+// or (g_each 0) one number a head at gate + t g_row + h g_head.
 int xi_head_linear(const void* x, long long x_row, long long x_head, const void* w, long long w_head, long long w_n,
                    long long w_k, void* out, long long o_row, long long o_head, const void* gate, long long g_row,
-                   long long g_head, int dtype, int n_tok, int H, int N, int K, hipStream_t stream) {
+                   long long g_head, int g_each, int dtype, int n_tok, int H, int N, int K, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && H > 0 && N > 0 && K > 0, "head_linear: bad sizes T=%d H=%d N=%d K=%d", n_tok, H, N, K);
   XI_CHECK(w_n == 1 || w_k == 1, "head_linear: the weight's outputs or its inputs must lie side by side");
   XI_CHECK(H <= 65535, "head_linear: too many heads");
@@ -297,20 +309,21 @@ int xi_head_linear(const void* x, long long x_row, long long x_head, const void*
     dim3 mgrid((unsigned)((n_tok + kHmRows - 1) / kHmRows), (unsigned)((N + kHmCols - 1) / kHmCols), (unsigned)H);
     // outputs (and the gate) in 8-byte pieces where every lane's 4 outputs start at one
     const int wide = o_row % 4 == 0 && o_head % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0 &&
-                     (gate == nullptr || (g_row % 4 == 0 && g_head % 4 == 0 && (reinterpret_cast<uintptr_t>(gate) & 7) == 0));
+                     (gate == nullptr || !g_each ||
+                      (g_row % 4 == 0 && g_head % 4 == 0 && (reinterpret_cast<uintptr_t>(gate) & 7) == 0));
     head_linear_mfma_kernel<<<mgrid, 256, 0, stream>>>((const bf16*)x, x_row, x_head, (const bf16*)w, w_head, w_n, (bf16*)out,
-                                                       o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N, K, wide);
+                                                       o_row, o_head, (const bf16*)gate, g_row, g_head, g_each, n_tok, N, K, wide);
     XI_LAUNCH_CHECK("head_linear");
     return 0;
   }
   if (dtype == kF32)
     head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)w, w_head, w_n, w_k,
-                                                        (float*)out, o_row, o_head, (const float*)gate, g_row, g_head, n_tok,
-                                                        N, K);
+                                                        (float*)out, o_row, o_head, (const float*)gate, g_row, g_head, g_each,
+                                                        n_tok, N, K);
   else if (dtype == kBF16)
     head_linear_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)x, x_row, x_head, (const bf16*)w, w_head, w_n, w_k,
-                                                       (bf16*)out, o_row, o_head, (const bf16*)gate, g_row, g_head, n_tok, N,
-                                                       K);
+                                                       (bf16*)out, o_row, o_head, (const bf16*)gate, g_row, g_head, g_each, n_tok,
+                                                       N, K);
   else
     XI_CHECK(false, "head_linear: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("head_linear");

@@ -11,6 +11,10 @@
 //            [E, 2F, H] (gate rows first), down [E, H, F]; or without a gate, y_e = Wd_e act(Wu_e x)
 //            with the up rows alone, [E, F, H].
 //   output   sum over the chosen experts, in the order they were chosen, of weight * y_e: float32.
+//   `scores` 2: the weights are sigmoid(z) of the chosen experts, as they are (the largest z are the largest scores).
+//   A weight may instead multiply the expert's INPUT, y_e = expert(weight * x) (`in_wt` of the gate/up product: the
+//   products are linear, so the weight multiplies their float32 sums before the activation; the down product then
+//   gets weights of 1).
 //
 // Every sum runs in an order fixed by the sizes alone (lanes stride over k, then the wave's
 // butterfly), so a token's result does not depend on the batch it is in.  The grouped
@@ -61,7 +65,7 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_kernel(const T* 
   }
   __syncthreads();
   if (wave != 0) return;
-  if (all_scores) {          // the softmax's maximum and denominator over every expert, in a fixed order
+  if (all_scores == 1) {     // the softmax's maximum and denominator over every expert, in a fixed order
     float m = -INFINITY;
     for (int e = lane; e < E; e += kWave) m = fmaxf(m, z[e]);
     m = wave_max(m);
@@ -101,7 +105,9 @@ __global__ __launch_bounds__(kRouteWaves* kWave) void moe_route_kernel(const T* 
     __builtin_amdgcn_s_waitcnt(0);      // lane 0's write to LDS is done before the wave reads z again
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane == 0 && all_scores) {
+  if (lane == 0 && all_scores == 2) {
+    for (int r = 0; r < top; ++r) wt[(size_t)t * top + r] = 1.f / (1.f + expf(-chosen[r]));
+  } else if (lane == 0 && all_scores) {
     const float m = denom_all[0], d = denom_all[1];
     float sum = 0.f;
     for (int r = 0; r < top; ++r) sum += expf(chosen[r] - m) / d;
@@ -127,10 +133,12 @@ constexpr int kMoeWaves = 4;
 template <typename T, int ACT, bool GATED>
 __global__ __launch_bounds__(kMoeWaves* kWave) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ wgu,
                                                                        const int* __restrict__ idx, T* __restrict__ mid,
-                                                                       int H, int F, int top, int FT) {
+                                                                       int H, int F, int top, int FT,
+                                                                       const float* __restrict__ in_wt) {
   extern __shared__ float xs[];
   const int pair = blockIdx.x, t = pair / top;
   const int e = idx[pair];
+  const float wi = in_wt ? in_wt[pair] : 1.f;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = to_float(x[(size_t)t * H + k]);
   __syncthreads();
@@ -164,8 +172,8 @@ __global__ __launch_bounds__(kMoeWaves* kWave) void moe_gate_up_kernel(const T* 
         if constexpr (GATED) au = fmaf(to_float(u[k]), xs[k], au);
       }
     }
-    ag = wave_sum(ag);
-    if constexpr (GATED) au = wave_sum(au);
+    ag = wave_sum(ag) * wi;
+    if constexpr (GATED) au = wave_sum(au) * wi;
     if (lane == 0) mid[(size_t)pair * F + f] = from_float<T>(GATED ? moe_act<ACT>(ag) * au : moe_act<ACT>(ag));
   }
 }
@@ -209,12 +217,13 @@ using namespace xi;
 extern "C" {
 
 // x [T, H] in `dtype`; wr float32 [E, H]; br float32 [E] or null; idx int32 [T, top]; wt float32 [T, top].
-// all_scores: see the head of the file.  extra float32 [T, X]: the products with rows E .. E + X - 1 of wr (X may be 0).
+// all_scores: 0, 1 (see the head of the file) or 2 (sigmoid of the chosen logits).  extra float32 [T, X]: the products with rows E .. E + X - 1 of wr (X may be 0).
 int xi_moe_route(const void* x, int dtype, const float* wr, const float* br, int* idx, float* wt, int n_tok, int H, int E,
                  int top, int all_scores, float* extra, int X, hipStream_t stream) {
   XI_CHECK(X >= 0 && (X == 0 || extra != nullptr), "moe_route: %d further rows need a place for their results", X);
   XI_CHECK(n_tok >= 0 && H > 0 && E > 0 && E <= kMaxExperts, "moe_route: bad sizes T=%d H=%d experts=%d (at most %d)", n_tok,
            H, E, kMaxExperts);
+  XI_CHECK(all_scores >= 0 && all_scores <= 2, "moe_route: unknown kind of scores %d", all_scores);
   XI_CHECK(top > 0 && top <= E && top <= kMaxTop, "moe_route: %d of %d experts cannot be chosen (at most %d)", top, E, kMaxTop);
   if (n_tok == 0) return 0;
   if (dtype == kF32)
@@ -231,8 +240,9 @@ int xi_moe_route(const void* x, int dtype, const float* wr, const float* br, int
 
 // x [T, H], wgu [E, 2F, H], idx [T * top] -> mid [T * top, F] = act(gate) * up, all in `dtype`;
 // gated 0: wgu [E, F, H] and mid = act(up).  act: 0 silu, 1 gelu (tanh form), 2 the square of relu.
+// in_wt float32 [T * top] or null: a weight a pair on the expert's input.
 int xi_moe_gate_up(const void* x, const void* wgu, const int* idx, void* mid, int dtype, int act, int gated, int n_tok, int H,
-                   int F, int E, int top, hipStream_t stream) {
+                   int F, int E, int top, const float* in_wt, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_gate_up: bad sizes T=%d H=%d F=%d E=%d top=%d", n_tok, H, F, E,
            top);
   XI_CHECK(act >= 0 && act <= 2, "moe_gate_up: unknown activation %d", act);
@@ -251,7 +261,7 @@ int xi_moe_gate_up(const void* x, const void* wgu, const int* idx, void* mid, in
       hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
       XI_CHECK(e_ == hipSuccess, "moe_gate_up: cannot get %zu bytes of LDS", lds);                              \
     }                                                                                                           \
-    kern<<<grid, kMoeWaves * kWave, lds, stream>>>((const TT*)x, (const TT*)wgu, idx, (TT*)mid, H, F, top, FT); \
+    kern<<<grid, kMoeWaves * kWave, lds, stream>>>((const TT*)x, (const TT*)wgu, idx, (TT*)mid, H, F, top, FT, in_wt); \
   } while (0)
 #define XI_GU_A(TT, G)            \
   do {                            \

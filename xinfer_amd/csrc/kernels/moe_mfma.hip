@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
                                                         const bf16* __restrict__ W, const int* __restrict__ tile_expert,
                                                         const int* __restrict__ tile_row0, const int* __restrict__ tile_rows,
                                                         const int* __restrict__ n_tiles, void* __restrict__ out, int N,
-                                                        int K) {
+                                                        int K, const float* __restrict__ in_wt) {
   constexpr bool GATED = FORM == 1, GATHER = FORM != 0;
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
@@ -136,15 +136,17 @@ __global__ __launch_bounds__(256) void moe_group_kernel(const bf16* __restrict__
     for (int v = 0; v < 4; ++v) {
       const int row = 16 * i + 4 * j + v;
       if (row >= rows) continue;
+      // a weight on the expert's INPUT: the products are linear, so it multiplies their sums before the activation
+      const float wi = (GATHER && in_wt) ? in_wt[order[row0 + row]] : 1.f;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const int col = nw0 + 16 * c + r;
         if (col >= N) continue;
         const size_t at = (size_t)(row0 + row) * N + col;
         if (GATED)
-          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]) * acc[i][GATED ? 2 + c : c][v]);
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(wi * acc[i][c][v]) * (wi * acc[i][GATED ? 2 + c : c][v]));
         else if (FORM == 2)
-          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]));
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(wi * acc[i][c][v]));
         else
           reinterpret_cast<float*>(out)[at] = acc[i][c][v];
       }
@@ -160,7 +162,8 @@ __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restri
                                                             const bf16* __restrict__ W, const int* __restrict__ tile_expert,
                                                             const int* __restrict__ tile_row0,
                                                             const int* __restrict__ tile_rows, const int* __restrict__ n_tiles,
-                                                            void* __restrict__ out, int N, int K) {
+                                                            void* __restrict__ out, int N, int K,
+                                                            const float* __restrict__ in_wt) {
   constexpr int MI = 8, BM = 128, LDA = 32 + 8;
   __shared__ __align__(16) bf16 As[2][BM * LDA];
   constexpr bool GATED = FORM == 1, GATHER = FORM != 0;
@@ -240,15 +243,17 @@ __global__ __launch_bounds__(256) void moe_group_lds_kernel(const bf16* __restri
     for (int v = 0; v < 4; ++v) {
       const int row = 16 * i + 4 * j + v;
       if (row >= rows) continue;
+      // a weight on the expert's INPUT: the products are linear, so it multiplies their sums before the activation
+      const float wi = (GATHER && in_wt) ? in_wt[order[row0 + row]] : 1.f;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const int col = nw0 + 16 * c + r;
         if (col >= N) continue;
         const size_t at = (size_t)(row0 + row) * N + col;
         if (GATED)
-          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]) * acc[i][GATED ? 2 + c : c][v]);
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(wi * acc[i][c][v]) * (wi * acc[i][GATED ? 2 + c : c][v]));
         else if (FORM == 2)
-          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(acc[i][c][v]));
+          reinterpret_cast<bf16*>(out)[at] = __float2bfloat16(moe_act_m<ACT>(wi * acc[i][c][v]));
         else
           reinterpret_cast<float*>(out)[at] = acc[i][c][v];
       }
@@ -286,10 +291,11 @@ int xi_moe_sort(const int* idx, int P, int E, int bm, int* order, int* slot_of, 
 // form 1 (gated): A = x [T, K] (row of a slot: order[slot] / top), W [E, 2N, K], out bfloat16 [P, N] = act(gate) * up;
 // form 2 (activated): the same rows, W [E, N, K], out bfloat16 [P, N] = act(up);
 // form 0 (plain): A [P, K] in slot order, W [E, N, K], out float32 [P, N].  K a multiple of 8.
-// act: 0 silu, 1 gelu (tanh form), 2 the square of relu.
+// act: 0 silu, 1 gelu (tanh form), 2 the square of relu.  in_wt (forms 1 and 2; null: none): float32 [P], a weight a pair
+// that multiplies the expert's input.
 int xi_moe_group(const void* A, const int* order, int top, const void* W, const int* tile_expert, const int* tile_row0,
                  const int* tile_rows, const int* n_tiles, int tiles_most, void* out, int N, int K, int bm, int form, int act,
-                 hipStream_t stream) {
+                 const float* in_wt, hipStream_t stream) {
   XI_CHECK(N > 0 && K > 0 && K % 8 == 0 && top > 0 && tiles_most > 0 && (bm == 32 || bm == 64 || bm == 128),
            "moe_group: bad sizes N=%d K=%d (a multiple of 8) top=%d tiles=%d rows=%d", N, K, top, tiles_most, bm);
   XI_CHECK(act >= 0 && act <= 2 && form >= 0 && form <= 2, "moe_group: unknown activation %d or form %d", act, form);
@@ -297,10 +303,10 @@ int xi_moe_group(const void* A, const int* order, int top, const void* W, const 
   XI_CHECK(grid.y <= 65535u, "moe_group: N=%d is too large", N);
 #define XI_MG(MI, G, ACT_)                                                                                            \
   moe_group_kernel<MI, G, ACT_><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,    \
-                                                          tile_row0, tile_rows, n_tiles, out, N, K)
+                                                          tile_row0, tile_rows, n_tiles, out, N, K, in_wt)
 #define XI_ML(G, ACT_)                                                                                                \
   moe_group_lds_kernel<G, ACT_><<<grid, 256, 0, stream>>>((const bf16*)A, order, top, (const bf16*)W, tile_expert,    \
-                                                          tile_row0, tile_rows, n_tiles, out, N, K)
+                                                          tile_row0, tile_rows, n_tiles, out, N, K, in_wt)
 #define XI_FORMS(LAUNCH, ...)                        \
   do {                                               \
     if (form == 0) LAUNCH(__VA_ARGS__ 0, 0);         \

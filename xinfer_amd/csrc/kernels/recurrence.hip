@@ -12,6 +12,10 @@
 //              bias[h]) (no clamp) from a column of the projection; the value row is multiplied by d_t as it is read
 //              (a selective state space: S <- a_t S + d_t k_t v_t^T).  Step size, exponentials and the product d_t v_t
 //              are float32.
+//   gates      a_t[i] = gates[t, h, 0] for every channel and the value row times gates[t, h, 1], both made
+//              beforehand (float32 [T, H, 2]: the keep and take factors of a matrix memory, mlstm.hip).
+// With `v_cols` < dv the value rows hold v_cols columns a head and the state's further columns read the value 1:
+// column v_cols of the state is then the sum of the (decayed, weighted) keys alone, the normalizer of a matrix memory.
 // With `group_heads` g > 1, q and k have one set of dk columns for every g heads (head h reads set h / g).
 // q, k and v are columns of a packed projection (a row stride and a column offset each); q and k are
 // multiplied by `q_scale` / `k_scale` in float32 as they are read.
@@ -56,8 +60,8 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k, long long k_stride, const T* __restrict__ v,
     long long v_stride, const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau,
     const float* __restrict__ head_decay, const T* __restrict__ step, long long step_stride,
-    const float* __restrict__ step_bias, const float* __restrict__ decay_log, int group_heads,
-    const float* __restrict__ state_in, long long in_stride, const long long* __restrict__ in_idx,
+    const float* __restrict__ step_bias, const float* __restrict__ decay_log, const float* __restrict__ gates, int v_cols,
+    int group_heads, const float* __restrict__ state_in, long long in_stride, const long long* __restrict__ in_idx,
     float* __restrict__ state_out, long long out_stride, const long long* __restrict__ out_idx,
     const int* __restrict__ first, const int* __restrict__ last, float* __restrict__ out, float* __restrict__ decay_out,
     int H, int dk, int dv, float q_scale, float k_scale) {
@@ -84,6 +88,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   const float sb = step ? step_bias[h] : 0.f, rate = step ? -expf(decay_log[h]) : 0.f;
   // the token's step size (1 where the decay has another source): every thread makes its own copy
   auto step_of = [&](int t) {
+    if (gates) return gates[((size_t)t * H + h) * 2 + 1];
     if (!step) return 1.f;
     const float x = to_float(step[(size_t)t * step_stride + h]) + sb;
     return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
@@ -94,13 +99,15 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
       fk = to_float(k[(size_t)t * k_stride + qk0 + c]) * k_scale;
       if (!ONE) fa = decay_of(z[((size_t)t * H + h) * dk + c] + zb, inv_tau);
     }
-    if (ONE) fa = step ? expf(rate * dt) : hd;
+    if (ONE) fa = gates ? gates[((size_t)t * H + h) * 2] : step ? expf(rate * dt) : hd;
   };
   float fq = 0.f, fk = 0.f, fa = 0.f;
   float dt = step_of(t0);
   fetch(t0, dt, fq, fk, fa);
   // the token's value is asked for a token ahead as well: no step of the walk waits for memory
-  float v_next = col ? to_float(v[(size_t)t0 * v_stride + h * dv + j]) * dt : 0.f;
+  // (a column past the value rows' own reads 1)
+  auto value_of = [&](int t) { return j < v_cols ? to_float(v[(size_t)t * v_stride + h * v_cols + j]) : 1.f; };
+  float v_next = col ? value_of(t0) * dt : 0.f;
   qs[0][c] = fq;
   ks[0][c] = fk;
   if (!ONE) as[0][c] = fa;
@@ -113,7 +120,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     if (t + 1 < t1) {
       dt = step_of(t + 1);
       fetch(t + 1, dt, fq, fk, fa);
-      if (col) v_next = to_float(v[(size_t)(t + 1) * v_stride + h * dv + j]) * dt;
+      if (col) v_next = value_of(t + 1) * dt;
     }
     float acc = 0.f;
     const float4* a4 = reinterpret_cast<const float4*>(&as[cur][wave * RPT]);
@@ -207,22 +214,24 @@ extern "C" {
 // q, k [T, .] with H dk columns from the given pointers (H / group_heads sets of dk columns if group_heads > 1), v with
 // H dv, rows `*_stride` elements apart, in `dtype`; the decay from z float32 [T, H dk] (z_bias float32 [H dk] or null), or
 // from head_decay float32 [H], or from step (rows of step_stride elements in `dtype`, H columns: the raw step sizes) with
-// step_bias and decay_log float32 [H]: one of the three.  Item w walks tokens
+// step_bias and decay_log float32 [H], or from gates float32 [T, H, 2] (the decay and the factor on the value row): one
+// of the four.  v_cols: the columns a head has in v's rows (dv, or fewer: the state's further columns read 1).  Item w walks tokens
 // first[w] .. last[w] - 1 from the state state_in + in_idx[w] * in_stride ([H, dk, dv] float32; in_idx null or a
 // negative entry: from zeros) and leaves its last state at state_out + out_idx[w] * out_stride (null or negative:
 // nowhere); out float32 [T, H, dv] or null (no results); decay_out float32 [items, H, dk] or null: the product of
 // each channel's decays over the item.
 int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k_stride, const void* v, long long v_stride,
                    int dtype, const float* z, const float* z_bias, float tau, const float* head_decay, const void* step,
-                   long long step_stride, const float* step_bias, const float* decay_log, int group_heads,
-                   const float* state_in,
+                   long long step_stride, const float* step_bias, const float* decay_log, const float* gates, int v_cols,
+                   int group_heads, const float* state_in,
                    long long in_stride, const long long* in_idx, float* state_out, long long out_stride,
                    const long long* out_idx, const int* first, const int* last, float* out, float* decay_out, int n_items, int H,
                    int dk, int dv, float q_scale, float k_scale, hipStream_t stream) {
   XI_CHECK(n_items >= 0 && H > 0 && dk > 0 && dv > 0, "linear_scan: bad sizes items=%d H=%d dk=%d dv=%d", n_items, H, dk, dv);
   XI_CHECK(dk <= kScanWaves * 64, "linear_scan: key heads of up to %d channels, not %d", kScanWaves * 64, dk);
-  XI_CHECK((z != nullptr) + (head_decay != nullptr) + (step != nullptr) == 1,
-           "linear_scan: a decay per token and channel, per head, or per token and head from a step size: one of them");
+  XI_CHECK((z != nullptr) + (head_decay != nullptr) + (step != nullptr) + (gates != nullptr) == 1,
+           "linear_scan: a decay per token and channel, per head, per token and head from a step size, or ready-made gates: one of them");
+  XI_CHECK(v_cols > 0 && v_cols <= dv, "linear_scan: %d value columns in rows for a state of %d", v_cols, dv);
   XI_CHECK(step == nullptr || (step_bias && decay_log && step_stride >= H), "linear_scan: a step size needs its bias and its rate");
   XI_CHECK(group_heads >= 1 && H % group_heads == 0, "linear_scan: %d heads in groups of %d", H, group_heads);
   XI_CHECK(z == nullptr || tau > 0.f, "linear_scan: tau must be positive");
@@ -237,7 +246,7 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
   const int rpt = (dk + kScanWaves - 1) / kScanWaves;
 #define XI_SCAN_ARGS(TT)                                                                                                      \
       (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, z, z_bias, inv_tau, head_decay, (const TT*)step,    \
-      step_stride, step_bias, decay_log, group_heads, state_in, in_stride,                                                    \
+      step_stride, step_bias, decay_log, gates, v_cols, group_heads, state_in, in_stride,                                                    \
       in_idx, state_out, out_stride, out_idx, first, last, out, decay_out, H, dk, dv, q_scale, k_scale
 #define XI_SCAN(TT, R)                                                                                                        \
   do {                                                                                                                        \

@@ -277,12 +277,13 @@ def scan_chunk_plan(q_lens, chunk: Optional[int] = None):
     return whole, long, chunks
 
 
-def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, group_heads,
+def _scan_launch(q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, gates, v_cols, group_heads,
                  state_in, in_stride, in_idx, state_out, out_stride, out_idx,
                  first, last, out, decay_out, items, H, dk, dv, q_scale, k_scale):
     _ok(lib().xi_linear_scan(_p(q), ctypes.c_longlong(qs), _p(k), ctypes.c_longlong(ks), _p(v), ctypes.c_longlong(vs),
                              _code(q, "linear_scan"), _p(z), _p(z_bias), ctypes.c_float(tau), _p(head_decay),
-                             _p(step), ctypes.c_longlong(ss), _p(step_bias), _p(decay_log), int(group_heads), _p(state_in),
+                             _p(step), ctypes.c_longlong(ss), _p(step_bias), _p(decay_log), _p(gates), int(v_cols),
+                             int(group_heads), _p(state_in),
                              ctypes.c_longlong(in_stride), _p(in_idx), _p(state_out), ctypes.c_longlong(out_stride),
                              _p(out_idx), ctypes.c_void_p(first), ctypes.c_void_p(last), _p(out), _p(decay_out), int(items),
                              H, dk, dv, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _stream()))
@@ -293,13 +294,17 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
                 tau: float = 1.0, head_decay: Optional[torch.Tensor] = None, q_scale: float = 1.0,
                 k_scale: float = 1.0, z_bias: Optional[torch.Tensor] = None, q_lens=None, plan_cache=None,
                 step: Optional[torch.Tensor] = None, step_bias: Optional[torch.Tensor] = None,
-                decay_log: Optional[torch.Tensor] = None, groups: Optional[int] = None) -> torch.Tensor:
+                decay_log: Optional[torch.Tensor] = None, groups: Optional[int] = None,
+                gates: Optional[torch.Tensor] = None, value_cols: Optional[int] = None) -> torch.Tensor:
     """Linear attention with a decaying float32 state per request and head, S <- diag(a) S + k v^T, o = S^T q,
     token by token from the state each request's slot holds (left there afterwards).  q, k [T, H dk] and
     v [T, H dv] may be column ranges of a packed projection.  The decay: `z` float32 [T, H dk], `z_bias`
     float32 [H dk] (or None) and `tau` (a = sigmoid(z + bias)^(1 / tau) per token and key channel) or `head_decay` float32 [H] (a constant per head),
     or `step` [T, H] (columns of a projection, in q's type), `step_bias` and `decay_log` float32 [H]: the step size d =
     softplus(step + step_bias), a = exp(-exp(decay_log) d) per token and head, and the token's value row times d.
+    Or `gates` float32 [T, H, 2], made beforehand: a = gates[t, h, 0] and the token's value row times gates[t, h, 1].
+    `value_cols` c < value_dim: v is [T, H c] and the state's columns from c on read the value 1 (column c then holds
+    the decayed sum of the weighted keys alone).
     `groups` G: q and k are [T, G dk] and head h reads the columns of group h // (H / G).
     state float32 [slots, H, dk, dv] (slots may be strided); state_slots int64 [B]; cu_q int32 [B + 1].
     Returns o float32 [T, H, dv].
@@ -313,11 +318,20 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     G = H if groups is None else int(groups)
     if G <= 0 or H % G:
         raise KernelError(f"linear_scan: {H} heads in {G} groups")
-    qs, ks, vs = _columns(q, G * dk, "linear_scan: q"), _columns(k, G * dk, "linear_scan: k"), _columns(v, H * dv, "linear_scan: v")
+    vc = dv if value_cols is None else int(value_cols)
+    if not (0 < vc <= dv):
+        raise KernelError(f"linear_scan: {vc} value columns for a state of {dv}")
+    qs, ks, vs = _columns(q, G * dk, "linear_scan: q"), _columns(k, G * dk, "linear_scan: k"), _columns(v, H * vc, "linear_scan: v")
     if k.shape[0] != T or v.shape[0] != T or q.dtype != k.dtype or q.dtype != v.dtype or not (q.device == k.device == v.device):
         raise KernelError("linear_scan: q, k and v must be rows of the same tokens, type and device")
-    _dev(z, head_decay, state_slots, cu_q, z_bias, step_bias, decay_log)
+    _dev(z, head_decay, state_slots, cu_q, z_bias, step_bias, decay_log, gates)
     ss = 0
+    if gates is not None:
+        if z is not None or head_decay is not None or step is not None:
+            raise KernelError("linear_scan: ready-made gates come alone")
+        _want(gates, torch.float32, "linear_scan: gates")
+        if tuple(gates.shape) != (T, H, 2) or not gates.is_contiguous():
+            raise KernelError(f"linear_scan: gates {tuple(gates.shape)} must be [{T}, {H}, 2]")
     if step is not None:
         if z is not None or head_decay is not None or step_bias is None or decay_log is None:
             raise KernelError("linear_scan: a step size comes with its bias and its rate, and alone")
@@ -330,9 +344,9 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
                 raise KernelError(f"linear_scan: {what} {tuple(t_.shape)} must be [{H}]")
     if z_bias is not None and (z is None or z_bias.dtype != torch.float32 or z_bias.shape != (H * dk,)):
         raise KernelError(f"linear_scan: the bias of the decay's logits must be float32 [{H * dk}], beside z")
-    if step is None and (z is None) == (head_decay is None):
+    if step is None and gates is None and (z is None) == (head_decay is None):
         raise KernelError("linear_scan: a decay per token (z) or per head (head_decay), one of them")
-    if step is not None:
+    if step is not None or gates is not None:
         pass
     elif z is not None:
         _want(z, torch.float32, "linear_scan: z")
@@ -355,7 +369,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
         raise KernelError("linear_scan: the portions' lengths do not add up to the step's tokens")
     out = torch.empty((T, H, dv), dtype=torch.float32, device=q.device)
     slot_stride = int(state.stride(0)) if state.shape[0] > 1 else H * dk * dv
-    common = (q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, H // G)
+    common = (q, k, v, qs, ks, vs, z, z_bias, tau, head_decay, step, ss, step_bias, decay_log, gates, vc, H // G)
     whole, long, chunks = scan_chunk_plan(q_lens) if q_lens is not None else (None, [], [])
     if not long:            # every request in one piece, straight from the step's own arrays
         _scan_launch(*common, state, slot_stride, state_slots, state, slot_stride, state_slots, cu_q.data_ptr(),
@@ -430,16 +444,26 @@ def head_norm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], eps: float, 
     return out
 
 
-def act_mul(gate_up: torch.Tensor, act: str = "silu") -> torch.Tensor:
-    """out = act(gate_up[:, :I]) * gate_up[:, I:] for an activation of `ACTIVATIONS` (float32 inside)."""
-    _dev(gate_up)
+def act_mul(gate_up: torch.Tensor, act: str = "silu", row_scale: Optional[torch.Tensor] = None,
+            row_of: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(gate_up[:, :I]) * gate_up[:, I:] for an activation of `ACTIVATIONS` (float32 inside).  `row_scale`
+    (float32; row t's factor is row_scale[row_of[t]], or row_scale[t] without `row_of` int32 [T]) multiplies gate and
+    up first: a factor on the input of the two products."""
+    _dev(gate_up, row_scale, row_of)
+    if row_scale is not None:
+        _want(row_scale, torch.float32, "act_mul: row_scale")
+        if row_of is not None:
+            _want(row_of, torch.int32, "act_mul: row_of")
+        if not row_scale.is_contiguous() or (row_of if row_of is not None else row_scale).numel() < gate_up.shape[0]:
+            raise KernelError("act_mul: a factor a row is needed")
     if act not in ACTIVATIONS:
         raise KernelError(f"act_mul: unknown activation {act!r} ({', '.join(ACTIVATIONS)})")
     if gate_up.dim() != 2 or gate_up.shape[1] % 2:
         raise KernelError("act_mul: input must be [T, 2I]")
     T, I = gate_up.shape[0], gate_up.shape[1] // 2
     out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
-    _ok(lib().xi_act_mul(_p(gate_up), _p(out), _code(gate_up, "act_mul"), ACTIVATIONS[act], T, I, _stream()))
+    _ok(lib().xi_act_mul(_p(gate_up), _p(out), _code(gate_up, "act_mul"), ACTIVATIONS[act], T, I, _p(row_scale),
+                         _p(row_of if row_scale is not None else None), _stream()))
     return out
 
 
@@ -542,7 +566,7 @@ def qkv_rows(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Opti
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int, all_scores: bool = False,
-              extra_rows: int = 0):
+              extra_rows: int = 0, sigmoid: bool = False):
     """Router of a mixture of experts: z = router @ x + bias in float32 (router float32 [E, H]), the `top`
     largest (ties: the lower index), weights = softmax over the chosen logits, or with `all_scores` the
     softmax over all experts, the chosen scores divided by their sum + 1e-20.  Returns
@@ -568,7 +592,7 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor
     wt = torch.empty((T, top), dtype=torch.float32, device=x.device)
     extra = torch.empty((T, X), dtype=torch.float32, device=x.device) if X else None
     _ok(lib().xi_moe_route(_p(x), _code(x, "moe_route"), _p(router), _p(bias), _p(idx), _p(wt), T, H, E, int(top),
-                           int(bool(all_scores)), _p(extra), X, _stream()))
+                           2 if sigmoid else int(bool(all_scores)), _p(extra), X, _stream()))
     return (idx, wt, extra) if X else (idx, wt)
 
 
@@ -588,12 +612,12 @@ MOE_LIBRARY_ROWS = 64     # rows an expert on average from which a step of porti
 
 
 def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
-                        act: str = "silu", gated: bool = True) -> torch.Tensor:
+                        act: str = "silu", gated: bool = True, weigh_input: bool = False) -> torch.Tensor:
     """`moe_experts` for steps of many tokens in bfloat16: the pairs sorted by expert on the device, the rows
     gathered in that order, and one plain product of the vendor library an expert and projection (as the
     dense feed-forward's products of many rows go to the library); the hand-written kernels do the sort,
     the activation and the combine.  Reads the experts' row counts on the host: for steps that bring
-    portions, which are never recorded into a graph."""
+    portions, which are never recorded into a graph.  `weigh_input`: see `moe_experts` (gated experts)."""
     _dev(x, gate_up, down, idx, wt)
     T, H = x.shape
     E, F2, _ = gate_up.shape
@@ -613,6 +637,11 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
     _ok(lib().xi_moe_sort(_p(idx), P, E, 128, _p(order), _p(slot_of), _p(ints[2 * P:2 * P + most]),
                           _p(ints[2 * P + most:2 * P + 2 * most]), _p(ints[2 * P + 2 * most:2 * P + 3 * most]),
                           _p(ints[2 * P + 3 * most:]), _stream()))
+    if weigh_input and not gated:
+        raise KernelError("moe_experts_library: a weight on the input is built for gated experts")
+    wt_in = wt.reshape(-1).contiguous() if weigh_input else None
+    if weigh_input:
+        wt = torch.ones_like(wt)
     counts = torch.bincount(idx.reshape(-1), minlength=E).tolist()          # the one read on the host
     rows = x.index_select(0, torch.div(order, top, rounding_mode="floor"))
     y = torch.empty((P, H), dtype=torch.float32, device=x.device)
@@ -620,7 +649,10 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
     for e, n in enumerate(counts[:E]):
         if n:
             mid = torch.nn.functional.linear(rows[at:at + n], gate_up[e])
-            mid = act_mul(mid, act) if gated else act_(mid, act)
+            if weigh_input:
+                mid = act_mul(mid, act, row_scale=wt_in, row_of=order[at:at + n])
+            else:
+                mid = act_mul(mid, act) if gated else act_(mid, act)
             torch.mm(mid, down[e].t(), out_dtype=torch.float32, out=y[at:at + n])
             at += n
     out = torch.empty((T, H), dtype=torch.float32, device=x.device)
@@ -630,13 +662,15 @@ def moe_experts_library(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tens
 
 def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, wt: torch.Tensor,
                 act: str = "silu", grouped: Optional[bool] = None, tile_rows: Optional[int] = None,
-                gated: bool = True) -> torch.Tensor:
+                gated: bool = True, weigh_input: bool = False) -> torch.Tensor:
     """sum over a token's chosen experts e (in the order of `idx`) of wt * down[e] @ (act(gate[e] @ x) * (up[e] @ x)):
     gate_up [E, 2F, H] (gate rows first), down [E, H, F], idx int32 / wt float32 [T, top].  Float32 [T, H].
     `gated` False: experts without a gate, wt * down[e] @ act(up[e] @ x), `gate_up` the up rows alone [E, F, H].
     One (token, expert) pair at a time, every sum in an order fixed by the sizes: the form of the
     float32 path and of steps with few tokens.  `grouped` (None: chosen by `moe_grouped_takes`): the pairs
-    sorted by expert on the device and each expert's rows multiplied in tiles on the matrix cores."""
+    sorted by expert on the device and each expert's rows multiplied in tiles on the matrix cores.
+    `weigh_input`: the weight multiplies the expert's input instead of its output, sum of expert_e(wt * x): it goes
+    onto the float32 sums of the gate and up products, before the activation."""
     _dev(x, gate_up, down, idx, wt)
     acts = ACTIVATIONS if gated else UNGATED_ACTIVATIONS
     if act not in acts:
@@ -655,6 +689,9 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
         raise KernelError("moe_experts: idx and weights must be [T, top]")
     top = int(idx.shape[1])
     out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    wt_in = None
+    if weigh_input:
+        wt_in, wt = wt.contiguous(), torch.ones_like(wt)
     if grouped is None:
         grouped = moe_grouped_takes(T, top, E, H, F, x.dtype)
     if grouped:
@@ -674,15 +711,16 @@ def moe_experts(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx:
         _ok(lib().xi_moe_sort(_p(idx), P, E, bm, _p(order), _p(slot_of), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), _stream()))
         mid = torch.empty((P, F), dtype=torch.bfloat16, device=x.device)
         _ok(lib().xi_moe_group(_p(x), _p(order), top, _p(gate_up), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(mid),
-                               F, H, bm, 1 if gated else 2, acts[act], _stream()))
+                               F, H, bm, 1 if gated else 2, acts[act], _p(wt_in), _stream()))
         y = torch.empty((P, H), dtype=torch.float32, device=x.device)
         _ok(lib().xi_moe_group(_p(mid), _p(order), top, _p(down), _p(t_e), _p(t_r0), _p(t_n), _p(n_tiles), most, _p(y),
-                               H, F, bm, 0, 0, _stream()))
+                               H, F, bm, 0, 0, None, _stream()))
         _ok(lib().xi_moe_combine(_p(y), _p(slot_of), _p(wt), _p(out), T, H, top, _stream()))
         return out
     mid = torch.empty((T * top, F), dtype=x.dtype, device=x.device)
     code = _code(x, "moe_experts")
-    _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, acts[act], int(bool(gated)), T, H, F, E, top, _stream()))
+    _ok(lib().xi_moe_gate_up(_p(x), _p(gate_up), _p(idx), _p(mid), code, acts[act], int(bool(gated)), T, H, F, E, top, _p(wt_in),
+                             _stream()))
     _ok(lib().xi_moe_down(_p(mid), _p(down), _p(idx), _p(wt), _p(out), code, T, H, F, E, top, _stream()))
     return out
 
@@ -743,13 +781,15 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
     return q_out
 
 
-def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what, dv=None):
+def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what, dv=None, key_heads=None):
     """K pool [pages, nkv, page, d]; V pool [pages, nkv, page, dv], or [pages, nkv, page / 8, dv, 8] if in
-    groups of eight keys (dv: the value head size, d unless given)."""
+    groups of eight keys (dv: the value head size, d unless given; `key_heads`: the K pool's heads where they are
+    not the V pool's)."""
     dv = d if dv is None else int(dv)
-    if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.dtype != dtype:
+    nkk = nkv if key_heads is None else int(key_heads)
+    if k_cache.dim() != 4 or k_cache.shape[1] != nkk or k_cache.shape[3] != d or k_cache.dtype != dtype:
         raise KernelError(f"{what}: K pool {tuple(k_cache.shape)} {k_cache.dtype} does not match "
-                          f"[pages, {nkv}, page_size, {d}] {dtype}")
+                          f"[pages, {nkk}, page_size, {d}] {dtype}")
     pages, _, page, _ = k_cache.shape
     if v_grouped and page % 8:
         raise KernelError(f"{what}: V in groups of eight keys needs pages of a multiple of 8 tokens, not {page}")
@@ -779,14 +819,17 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     T, nq, d = q.shape
     if k_cache.dim() != 4:
         raise KernelError("attention: the K pool must be [pages, nkv, page_size, d]")
-    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    nkk, page = int(k_cache.shape[1]), k_cache.shape[2]
+    nkv = nkk if v_cache is None else int(v_cache.shape[1])       # the K pool may hold fewer heads than the V pool
+    if nkk <= 0 or nkv <= 0 or nq % nkk or nq % nkv:
+        raise KernelError(f"attention: {nq} query heads on {nkk} key heads and {nkv} value heads")
     if v_cache is None:
         dv = int(value_dim or 0)
         if not (0 < dv <= d) or v_grouped or k_cache.shape[3] != d or k_cache.dtype != q.dtype:
             raise KernelError(f"attention: values inside the keys need 0 < value_dim <= {d} and a pool [pages, nkv, page, {d}]")
     else:
         dv = int(v_cache.shape[3])
-        _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention", dv=dv)
+        _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention", dv=dv, key_heads=nkk)
     if sinks is not None:
         _want(sinks, torch.float32, "attention: sinks")
         if sinks.shape != (nq,):
@@ -809,7 +852,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
         int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
         int(window), int(page), T, nq, nkv, d, dv, int(bool(v_grouped)), ctypes.c_float(softcap), _p(slopes), _p(sinks),
-        int(v_cache is None), _stream()))
+        int(v_cache is None), nkk, _stream()))
     return out
 
 
@@ -1042,7 +1085,9 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
     of its one new token, all at its last position, `cu_q` counts rows, `sinks` is [H] and blocks may hold many rows."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes, sinks)
     T, nq, d = q.shape
-    nkv, page, dv = k_cache.shape[1], k_cache.shape[2], int(vt_cache.shape[3])
+    nkk, nkv, page, dv = int(k_cache.shape[1]), int(vt_cache.shape[1]), k_cache.shape[2], int(vt_cache.shape[3])
+    if nkk <= 0 or nkv % nkk:
+        raise KernelError(f"attention_biased: {nkv} kv heads on {nkk} key heads")
     _want(q, torch.bfloat16, "attention_biased: q")
     if sinks is not None:
         _want(sinks, torch.float32, "attention_biased: sinks")
@@ -1050,7 +1095,7 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
             raise KernelError(f"attention_biased: sinks {tuple(sinks.shape)} must be one a query head, [{int(rows_heads) or nq}]")
     if rows_heads and (nq != 1 or nkv != 1 or slopes is not None or T % int(rows_heads)):
         raise KernelError("attention_biased: rows that are a token's heads come with one head, no slopes and whole tokens")
-    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv)
+    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv, key_heads=nkk)
     for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
         _want(t, torch.int32, f"attention_biased: {name}")
     B = ctx_lens.shape[0]
@@ -1081,7 +1126,7 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
         _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), _p(sinks), int(window),
         int(page), nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), int(rows_heads),
-        _stream()))
+        nkk, _stream()))
     return out
 
 
@@ -1182,12 +1227,13 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     matrix-core kernels of their own (`attention_biased_bf16`).  `v_cache` None: a key's first
     `value_dim` dims are its value, which only the generic kernel reads that way."""
     T, nq, d = q.shape
-    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    nkk, page = int(k_cache.shape[1]), k_cache.shape[2]
+    nkv = nkk if v_cache is None else int(v_cache.shape[1])      # the K pool may hold fewer heads (see `attention_generic`)
     bt = ctx.block_tables[group]
     if v_cache is None:
         return attention_generic(q, k_cache, None, bt, ctx.tok_seq, ctx.positions, scale, window, softcap=softcap,
                                  slopes=slopes, sinks=sinks, value_dim=value_dim)
-    if softcap > 0 or slopes is not None or sinks is not None or v_cache.shape[3] != d:
+    if softcap > 0 or slopes is not None or sinks is not None or v_cache.shape[3] != d or nkk != nkv:
         dv = int(v_cache.shape[3])
         if q.dtype == torch.bfloat16 and v_grouped and BIASED_MFMA and attention_biased_supported(nq, nkv, d, dv, page):
             if ctx.max_q_len == 1 and nkv == 1 and nq >= HEAD_ROWS_FROM and slopes is None and q.is_contiguous():
@@ -1755,18 +1801,22 @@ def head_rows(qkv: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_c
 def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight: torch.Tensor, eps: float,
                 slots: torch.Tensor, pool: torch.Tensor, q_full: torch.Tensor, heads: int, dim: int, rot_dim: int,
                 rank: int, cos: torch.Tensor, sin: torch.Tensor, interleaved: bool, positions: torch.Tensor,
-                values: Optional[torch.Tensor] = None) -> None:
+                values: Optional[torch.Tensor] = None, q_rows: Optional[torch.Tensor] = None) -> None:
     """From the packed projection `proj` [T, W] (the heads' q parts [H, dim + rot_dim] from column `q_offset`, the down
     projection [rank + rot_dim] from `down_offset`): the latent = RMSNorm(down[:rank]) * norm_weight and the turned
     down[rank:] into `pool` [pages, 1, page, rank + rot_dim] at `slots`; every head's turned q part into
     q_full[:, h, rank:] (q_full [T, H, rank + rot_dim]).  `values` [pages, 1, page / 8, rank, 8]: the latent once
-    more, in groups of eight tokens, as the matrix-core attention kernels read values."""
-    _dev(proj, norm_weight, slots, pool, q_full, cos, sin, positions, values)
+    more, in groups of eight tokens, as the matrix-core attention kernels read values.  `q_rows` [T, >= q_offset +
+    H (dim + rot_dim)]: the heads' q parts are rows of this tensor instead of `proj`'s."""
+    _dev(proj, norm_weight, slots, pool, q_full, cos, sin, positions, values, q_rows)
     H, d, r, rank = int(heads), int(dim), int(rot_dim), int(rank)
     if proj.dim() != 2 or q_full.dtype != proj.dtype or pool.dtype != proj.dtype:
         raise KernelError("latent_rows: the projection, the pool and q of one type")
     T, W = proj.shape
-    if q_offset < 0 or down_offset < 0 or q_offset + H * (d + r) > W or down_offset + rank + r > W:
+    if q_rows is not None and (q_rows.dim() != 2 or q_rows.shape[0] != T or q_rows.dtype != proj.dtype or q_rows.stride(1) != 1):
+        raise KernelError("latent_rows: the q parts must be rows of the same tokens and type")
+    QW = W if q_rows is None else int(q_rows.shape[1])
+    if q_offset < 0 or down_offset < 0 or q_offset + H * (d + r) > QW or down_offset + rank + r > W:
         raise KernelError(f"latent_rows: rows of {W} do not hold the q parts and the down projection")
     if tuple(q_full.shape) != (T, H, rank + r) or pool.dim() != 4 or pool.shape[1] != 1 or pool.shape[3] != rank + r:
         raise KernelError(f"latent_rows: q {tuple(q_full.shape)} must be [{T}, {H}, {rank + r}], the pool [pages, 1, page, {rank + r}]")
@@ -1783,12 +1833,13 @@ def latent_rows(proj: torch.Tensor, q_offset: int, down_offset: int, norm_weight
         raise KernelError(f"latent_rows: the values' pool {tuple(values.shape)} must be [{pool.shape[0]}, 1, page / 8, {rank}, 8]")
     _ok(lib().xi_latent_rows(_p(proj), ctypes.c_longlong(W), int(q_offset), int(down_offset), _code(proj, "latent_rows"),
                              _p(norm_weight), ctypes.c_float(eps), _p(slots), _p(pool), _p(values), int(pool.shape[2]), _p(q_full), T, H,
-                             d, r, rank, _p(cos), _p(sin), int(bool(interleaved)), _p(positions), _stream()))
+                             d, r, rank, _p(cos), _p(sin), int(bool(interleaved)), _p(positions), _p(q_rows),
+                             ctypes.c_longlong(0 if q_rows is None else (int(q_rows.stride(0)) if T > 1 else QW)), _stream()))
 
 
 def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, h, n] = sum_k x[t, h, k] * w[h, n, k] for every head, float32 sums; with `gate`
-    [T, H, N], out *= sigmoid(gate).  bfloat16 operands whose K is contiguous in whole 16-byte chunks run on the
+    [T, H, N], out *= sigmoid(gate); a gate [T, H] is one number a head.  bfloat16 operands whose K is contiguous in whole 16-byte chunks run on the
     matrix cores; others, and float32, on the vector units in ascending k.  All operands may be strided views ([T, H, .] of packed rows; w [H, N, K] with
     either N or K contiguous) of one type; `out` [T, H, N] is written in place."""
     for t in (x, w, out, gate):
@@ -1798,15 +1849,17 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optio
         raise KernelError("head_linear: x [T, H, K], w [H, N, K], out [T, H, N]")
     T, H, K = x.shape
     N = w.shape[1]
-    if tuple(w.shape) != (H, N, K) or tuple(out.shape) != (T, H, N) or (gate is not None and tuple(gate.shape) != (T, H, N)):
+    each = gate is None or gate.dim() == 3
+    if (tuple(w.shape) != (H, N, K) or tuple(out.shape) != (T, H, N)
+            or (gate is not None and tuple(gate.shape) != ((T, H, N) if each else (T, H)))):
         raise KernelError(f"head_linear: x {tuple(x.shape)}, w {tuple(w.shape)} and out {tuple(out.shape)} do not match")
-    if x.stride(2) != 1 or out.stride(2) != 1 or (gate is not None and gate.stride(2) != 1) or 1 not in (w.stride(1), w.stride(2)):
+    if x.stride(2) != 1 or out.stride(2) != 1 or (gate is not None and each and gate.stride(2) != 1) or 1 not in (w.stride(1), w.stride(2)):
         raise KernelError("head_linear: the last axis of x, out and the gate, and N or K of w, must be contiguous")
     ll = ctypes.c_longlong
     g = gate if gate is not None else out
     _ok(lib().xi_head_linear(_p(x), ll(x.stride(0)), ll(x.stride(1)), _p(w), ll(w.stride(0)), ll(w.stride(1)), ll(w.stride(2)),
                              _p(out), ll(out.stride(0)), ll(out.stride(1)), _p(gate), ll(g.stride(0)), ll(g.stride(1)),
-                             _code(x, "head_linear"), T, H, N, K, _stream()))
+                             int(each), _code(x, "head_linear"), T, H, N, K, _stream()))
     return out
 
 
@@ -1880,4 +1933,152 @@ def gated_group_norm(y: torch.Tensor, x: torch.Tensor, skip: torch.Tensor, z: to
     out = torch.empty((T, W), dtype=out_dtype, device=y.device)
     _ok(lib().xi_gated_group_norm(_p(y), _p(x), ctypes.c_longlong(xs), _p(skip), _p(z), ctypes.c_longlong(zs), _p(weight),
                                   ctypes.c_float(eps), _p(out), _code(out, "gated_group_norm"), T, W, dv, int(groups), _stream()))
+    return out
+
+
+# ---- around the state of a matrix memory ----------------------------------------------------------------------------
+def mlstm_gates(z: torch.Tensor, bias: torch.Tensor, cap: float, m_state: torch.Tensor, state_slots: torch.Tensor,
+                cu_q: torch.Tensor, heads: int):
+    """The gates of a matrix memory for a step's tokens.  z float32 [T, 2 H] (rows may be a column range): the input
+    gate's logits, then the forget gate's; bias float32 [2 H]; log_in = cap tanh((z_i + b_i) / cap), log_keep =
+    logsigmoid(cap tanh((z_f + b_f) / cap)); the running maximum m' = max(log_keep + m, log_in) is walked token by token
+    from m_state float32 [slots, H] (left there afterwards).  Returns gates float32 [T, H, 2] = (exp(log_keep + m - m'),
+    exp(log_in - m')) and floor float32 [T, H] = exp(-m')."""
+    _dev(bias, state_slots, cu_q)
+    H = int(heads)
+    _want(z, torch.float32, "mlstm_gates: z")
+    _want(bias, torch.float32, "mlstm_gates: bias")
+    _want(m_state, torch.float32, "mlstm_gates: m_state")
+    _want(state_slots, torch.int64, "mlstm_gates: state_slots")
+    _want(cu_q, torch.int32, "mlstm_gates: cu_q")
+    zs = _columns(z, 2 * H, "mlstm_gates: z")
+    T, B = z.shape[0], state_slots.shape[0]
+    if bias.shape != (2 * H,) or cu_q.shape != (B + 1,) or m_state.dim() != 2 or m_state.shape[1] != H or m_state.stride(1) != 1:
+        raise KernelError(f"mlstm_gates: bias [{2 * H}], cu_q [B + 1], m_state [slots, {H}] expected")
+    gates = torch.empty((T, H, 2), dtype=torch.float32, device=z.device)
+    floor = torch.empty((T, H), dtype=torch.float32, device=z.device)
+    stride = int(m_state.stride(0)) if m_state.shape[0] > 1 else H
+    _ok(lib().xi_mlstm_gates(_p(z), ctypes.c_longlong(zs), _p(bias), ctypes.c_float(cap), _p(m_state), ctypes.c_longlong(stride),
+                             _p(state_slots), _p(cu_q), _p(gates), _p(floor), int(B), H, _stream()))
+    return gates, floor
+
+
+def mlstm_finish(o: torch.Tensor, floor: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """o float32 [T, H, dv + 1] (a matrix memory's results; the last column is n . q): y = o[:dv] / (max(|o[dv]|, floor) +
+    1e-6), each head of y divided by its root mean square over dv (eps inside the root), times `weight` float32 [H dv],
+    times sigmoid(gate) (gate [T, H dv], may be a column range of a packed projection, in `out_dtype`).  Returns
+    [T, H dv] in `out_dtype`."""
+    _dev(o, floor, weight)
+    _want(o, torch.float32, "mlstm_finish: o")
+    _want(floor, torch.float32, "mlstm_finish: floor")
+    _want(weight, torch.float32, "mlstm_finish: weight")
+    if o.dim() != 3 or o.shape[2] < 2 or not o.is_contiguous():
+        raise KernelError("mlstm_finish: o must be [T, H, dv + 1]")
+    T, H, dv = o.shape[0], o.shape[1], o.shape[2] - 1
+    gs = _columns(gate, H * dv, "mlstm_finish: gate")
+    if (gate.shape[0] != T or gate.dtype != out_dtype or gate.device != o.device or tuple(floor.shape) != (T, H)
+            or not floor.is_contiguous() or weight.shape != (H * dv,)):
+        raise KernelError(f"mlstm_finish: gate rows of the same tokens in the output's type, floor [T, H], weight [{H * dv}]")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    _ok(lib().xi_mlstm_finish(_p(o), _p(floor), _p(weight), ctypes.c_float(eps), _p(gate), ctypes.c_longlong(gs), _p(out),
+                              _code(out, "mlstm_finish"), T, H, dv, _stream()))
+    return out
+
+
+# ---- rows of an attention with a short convolution and mixed heads -----------------------------------------------------
+def conv_qkv_rows(qkv: torch.Tensor, conv_weight: Optional[torch.Tensor], tails: Optional[torch.Tensor],
+                  state_slots: torch.Tensor, tok_seq: torch.Tensor, cu_q: torch.Tensor, q_weight: Optional[torch.Tensor],
+                  k_weight: Optional[torch.Tensor], eps: float, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, v_grouped: bool = False,
+                  value_unit_norm: bool = False, talk: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The first nq d + nkv d + nkv dv columns of a packed projection made ready for attention: a causal convolution per
+    channel over the last `taps` tokens (`conv_weight` float32 [C, taps]; None: none; inputs from before the step come
+    from `tails` float32 [slots, taps - 1, C] at `state_slots`, which `conv_tail` moves on afterwards), RMSNorm over the
+    whole q part and the whole k part (weights float32; None: none), every value head divided by its root mean square
+    (`value_unit_norm`), k and v into the paged cache at `slots`.  With `talk` float32 [nq, nq] (head h's score is
+    sum_g talk[h, g] (q_g . k)) the sum is taken on the query's side: the result is q' [T, nq, nkv d] and the K pool
+    [pages, 1, page, nkv d] holds a token's whole k row as one head; without, q [T, nq, d] and a K pool [pages, nkv, page, d]."""
+    _dev(conv_weight, state_slots, tok_seq, cu_q, q_weight, k_weight, slots, k_cache, v_cache, talk)
+    nq, nkv, d, dv = int(num_heads), int(num_kv_heads), int(head_dim), int(value_dim)
+    C = nq * d + nkv * d + nkv * dv
+    if qkv.dim() != 2 or qkv.shape[1] < C or qkv.stride(1) != 1:
+        raise KernelError(f"conv_qkv_rows: rows {tuple(qkv.shape)} do not hold {C} channels")
+    T = qkv.shape[0]
+    stride = int(qkv.stride(0)) if T > 1 else int(qkv.shape[1])
+    taps = 1
+    tail_stride = 0
+    if conv_weight is not None:
+        _want(conv_weight, torch.float32, "conv_qkv_rows: the convolution's weight")
+        if conv_weight.dim() != 2 or conv_weight.shape[0] != C or not conv_weight.is_contiguous():
+            raise KernelError(f"conv_qkv_rows: the convolution's weight {tuple(conv_weight.shape)} must be [{C}, taps]")
+        taps = int(conv_weight.shape[1])
+    if taps > 1:
+        if tails is None:
+            raise KernelError("conv_qkv_rows: a convolution needs the requests' tails")
+        _want(tails, torch.float32, "conv_qkv_rows: tails")
+        _want(state_slots, torch.int64, "conv_qkv_rows: state_slots")
+        _want(tok_seq, torch.int32, "conv_qkv_rows: tok_seq")
+        _want(cu_q, torch.int32, "conv_qkv_rows: cu_q")
+        if tails.dim() != 3 or tuple(tails.shape[1:]) != (taps - 1, C) or tails[0].stride() != (C, 1) or tok_seq.shape != (T,):
+            raise KernelError(f"conv_qkv_rows: tails {tuple(tails.shape)} must be [slots, {taps - 1}, {C}] with whole slots")
+        tail_stride = int(tails.stride(0)) if tails.shape[0] > 1 else (taps - 1) * C
+    for w, n in ((q_weight, nq * d), (k_weight, nkv * d)):
+        if w is not None:
+            _want(w, torch.float32, "conv_qkv_rows: norm weight")
+            if w.shape != (n,):
+                raise KernelError(f"conv_qkv_rows: norm weight {tuple(w.shape)} is not [{n}]")
+    if (q_weight is None) != (k_weight is None):
+        raise KernelError("conv_qkv_rows: q and k norm weights come together")
+    _want(slots, torch.int64, "conv_qkv_rows: slots")
+    if slots.shape != (T,):
+        raise KernelError("conv_qkv_rows: slots must be [T]")
+    if talk is not None:
+        _want(talk, torch.float32, "conv_qkv_rows: talk")
+        if tuple(talk.shape) != (nq, nq) or not talk.is_contiguous():
+            raise KernelError(f"conv_qkv_rows: talk {tuple(talk.shape)} must be [{nq}, {nq}]")
+        _check_cache(k_cache, v_cache, nkv, nkv * d, qkv.dtype, v_grouped, "conv_qkv_rows", dv=dv, key_heads=1)
+        q_out = torch.empty((T, nq, nkv * d), dtype=qkv.dtype, device=qkv.device)
+    else:
+        _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_grouped, "conv_qkv_rows", dv=dv)
+        q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
+    _ok(lib().xi_conv_qkv_rows(_p(qkv), ctypes.c_longlong(stride), _code(qkv, "conv_qkv_rows"), _p(conv_weight), taps,
+                               _p(tails if taps > 1 else None), ctypes.c_longlong(tail_stride),
+                               _p(state_slots if taps > 1 else None), _p(tok_seq if taps > 1 else None),
+                               _p(cu_q if taps > 1 else None), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
+                               int(bool(value_unit_norm)), _p(talk), _p(slots), _p(q_out), _p(k_cache), _p(v_cache),
+                               int(k_cache.shape[2]), T, nq, nkv, d, dv, int(bool(v_grouped)), _stream()))
+    return q_out
+
+
+def head_gate_(x: torch.Tensor, gate: torch.Tensor, heads: int) -> torch.Tensor:
+    """x [T, H dv] *= sigmoid(gate[t, h]) head by head, in place; gate [T, H] may be a column range of a packed
+    projection, in x's type."""
+    _dev(x)
+    H = int(heads)
+    if x.dim() != 2 or x.shape[1] % H or not x.is_contiguous():
+        raise KernelError(f"head_gate: x {tuple(x.shape)} is not [T, {H} dv]")
+    gs = _columns(gate, H, "head_gate: gate")
+    if gate.shape[0] != x.shape[0] or gate.dtype != x.dtype or gate.device != x.device:
+        raise KernelError("head_gate: the gate must be rows of the same tokens in x's type")
+    _ok(lib().xi_head_gate(_p(x), _p(gate), ctypes.c_longlong(gs), _code(x, "head_gate"), int(x.shape[0]), H, int(x.shape[1]) // H,
+                           _stream()))
+    return x
+
+
+def rows_rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """x [T, n] (rows may be a column range of a packed projection, float32 or bfloat16) -> x * rsqrt(mean(x^2) + eps) *
+    weight (float32 [n]; None: no weight) in `out_dtype`; float32 inside."""
+    _dev(weight)
+    if x.dim() != 2 or x.stride(1) != 1 or not x.is_cuda:
+        raise KernelError(f"rows_rmsnorm: {tuple(x.shape)} with strides {x.stride()} is not rows")
+    T, n = x.shape
+    if weight is not None:
+        _want(weight, torch.float32, "rows_rmsnorm: weight")
+        if weight.shape != (n,):
+            raise KernelError(f"rows_rmsnorm: weight {tuple(weight.shape)} is not [{n}]")
+    out = torch.empty((T, n), dtype=out_dtype, device=x.device)
+    stride = int(x.stride(0)) if T > 1 else n
+    _ok(lib().xi_rows_rmsnorm(_p(x), ctypes.c_longlong(stride), _code(x, "rows_rmsnorm"), _p(weight), ctypes.c_float(eps), _p(out),
+                              _code(out, "rows_rmsnorm"), int(T), int(n), _stream()))
     return out

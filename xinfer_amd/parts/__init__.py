@@ -4,6 +4,6 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Blo
                    Stream, block_class, feed_forward_class, mixer_class, norm_class,
                    position_encoding_class, register_block, register_feed_forward,
                    register_mixer, register_norm, register_position_encoding)
-from . import attention, block, latent, mlp, moe, norm, parallel, recurrent, rope, ssm, stream_ops  # noqa: F401  (register the built-in kinds)
+from . import attention, block, latent, mlp, mlstm, moe, norm, parallel, recurrent, rope, ssm, stream_ops  # noqa: F401  (register the built-in kinds)
 from .embedding import Embedding, LMHead
 from .linear import Linear

@@ -24,6 +24,17 @@ root), without a weight, AFTER the rotation.  A rotation turns pairs of dims and
 is, so the plain form computes this with its own kernels (norm with a weight of ones, then rotation: the same but for
 rounding); with the options of the paragraph above, or with `general=True`, a kernel that takes a head at a time does
 it in the order given (`kernels.head_rows`: rotation of either pairing, then the unit norm, then the cache write).
+
+A third group of options, each a parameter of the spec, goes through `_forward_rows` (no rotation, `qk_norm` "row" or
+none): `conv` n > 1: q, k and v pass a causal convolution per channel over the last n tokens right after the
+projection (tensors `q_conv`, `k_conv`, `v_conv` [channels, n], no bias; the last n - 1 projected rows of a request are
+state of the layer, "conv_tail"); `value_norm="head_unit"`: every value head is divided by its root mean square and
+cached so; `talking_heads`: head h's score of a key is sum_g talk[h, g] * (head g's score) before the softmax (tensor
+`talk` [heads, heads]); `head_gate`: head h's result times sigmoid(w_h . x), one number a head (tensor `head_gate`
+[heads, hidden], packed with q, k and v).  The heads' sum moves to the query's side, q'_h = [sum_{g on kv head c}
+talk[h, g] q_g for every kv head c], scored against a token's whole k row: the K pool of such a layer holds one head
+of kv_heads * head_dim dims and the attention kernels read the keys of that one head and the values of the query head's
+own kv head.
 """
 from __future__ import annotations
 
@@ -34,7 +45,7 @@ import torch
 from .. import kernels
 from ..config.spec import PartSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import (Folded, KVNeed, LayerCache, Mixer, StepContext, position_encoding_class,
+from .base import (Folded, KVNeed, LayerCache, Mixer, PAGE, PoolNeed, StateNeed, StepContext, position_encoding_class,
                    register_mixer)
 from .linear import Linear
 
@@ -78,6 +89,21 @@ class PagedAttention(Mixer):
         if self.by_head and (self.row_norm or self.value_mix_key is not None):
             raise NotImplementedError("attention whose heads are normed one by one or turned in pairs (2i, 2i + 1) takes no "
                                       "norm over the whole projection and no blended values")
+        self.taps = int(spec.get("conv") or 0)
+        self.value_unit = spec.get("value_norm") == "head_unit"
+        if spec.get("value_norm") not in (None, "head_unit"):
+            raise ValueError(f"value_norm {spec.get('value_norm')!r}: 'head_unit' or none")
+        self.talking = bool(spec.get("talking_heads", False))
+        self.head_gate = bool(spec.get("head_gate", False))
+        # a convolution, normed values, mixed heads or a gate a head: one kernel makes a token's row ready
+        self.rows_form = self.taps > 1 or self.value_unit or self.talking or self.head_gate
+        if self.rows_form:
+            self.general = True
+            if (self.by_head or spec.get("position") is not None or self.softcap > 0 or self.slope_values is not None
+                    or self.value_mix_key is not None or self.bias or (self.qk_norm and not self.row_norm)):
+                raise NotImplementedError("attention with a convolution, normed values, mixed heads or a gate a head takes the "
+                                          "q/k norm over the whole projection or none, and no rotation, cap, bias or blend")
+        self.conv_w = self.talk = None
         if self.general and not self.by_head and spec.get("position") is not None and self.qk_norm:
             raise NotImplementedError("attention with a soft cap, a distance bias, blended values or another value size takes a "
                                       "rotation of the pairs (i, i + rotary_dim / 2) and then no q/k norm")
@@ -103,7 +129,9 @@ class PagedAttention(Mixer):
     # ---- weights -----------------------------------------------------------
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix",
+             "q_conv": "q_conv.weight", "k_conv": "k_conv.weight", "v_conv": "v_conv.weight", "talk": "talk",
+             "head_gate": "head_gate.weight"}
 
     @classmethod
     def _names(cls, spec: PartSpec, prefix: str):
@@ -128,6 +156,14 @@ class PagedAttention(Mixer):
         vm = spec.get("value_mix")
         if vm and not vm.get("source", False):
             out.append(TensorDecl(n["value_mix"], (), "mix"))
+        taps = int(spec.get("conv") or 0)
+        if taps > 1:
+            out += [TensorDecl(n["q_conv"], (nq * d, taps), "normal(0,0.5)"), TensorDecl(n["k_conv"], (nkv * d, taps), "normal(0,0.5)"),
+                    TensorDecl(n["v_conv"], (nkv * dv, taps), "normal(0,0.5)")]
+        if spec.get("talking_heads", False):
+            out.append(TensorDecl(n["talk"], (nq, nq), "normal(0,0.5)"))
+        if spec.get("head_gate", False):
+            out.append(TensorDecl(n["head_gate"], (nq, h)))
         return out
 
     def load(self, store: WeightStore, prefix: str, device) -> None:
@@ -135,7 +171,11 @@ class PagedAttention(Mixer):
             t = store.get(name, None, device)
             return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
         names = self._names(self.spec, prefix)
-        parts = [lin(names[n]) for n in ("q", "k", "v")]
+        parts = [lin(names[n]) for n in (("q", "k", "v", "head_gate") if self.head_gate else ("q", "k", "v"))]
+        if self.taps > 1:
+            self.conv_w = torch.cat([store.get(names[n], torch.float32, device) for n in ("q_conv", "k_conv", "v_conv")]).contiguous()
+        if self.talking:
+            self.talk = store.get(names["talk"], torch.float32, device).contiguous()
         common = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
         self.qkv = Linear(torch.cat([p.to(common) for p in parts], dim=0))
         self.o = Linear(lin(names["o"]))
@@ -157,8 +197,16 @@ class PagedAttention(Mixer):
     # ---- cache ---------------------------------------------------------------
     def cache_need(self) -> KVNeed:
         # the matrix-core kernels of the bfloat16 path read V in groups of eight keys
-        return KVNeed.keys_values(self.nkv, self.d, self.window, v_grouped=self.dtype == torch.bfloat16,
+        need = KVNeed.keys_values(self.nkv, self.d, self.window, v_grouped=self.dtype == torch.bfloat16,
                                   value_dim=self.dv)
+        if self.talking:           # mixed heads score against a token's whole k row: one key head of all kv heads' dims
+            need = KVNeed(need.window, (PoolNeed("k", (1, PAGE, self.nkv * self.d)), need.pools[1]))
+        return need
+
+    def state_need(self):
+        if self.taps > 1:
+            return StateNeed((self.taps - 1, self.nq * self.d + self.nkv * (self.d + self.dv)), torch.float32, "conv_tail")
+        return None
 
     # ---- step ----------------------------------------------------------------
     takes_sink = True
@@ -204,6 +252,8 @@ class PagedAttention(Mixer):
 
     def _forward_general(self, x, ctx: StepContext, cache: LayerCache, sink=None):
         """The step with the options of the module's second paragraph (no rotation)."""
+        if self.rows_form:
+            return self._forward_rows(x, ctx, cache)
         qkv = self.qkv(x, out_dtype=self.dtype)
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
         vt = self.dtype == torch.bfloat16
@@ -233,3 +283,24 @@ class PagedAttention(Mixer):
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt,
                               softcap=self.softcap, slopes=self.slopes)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)
+
+    def _forward_rows(self, x, ctx: StepContext, cache: LayerCache):
+        """The step with the options of the module's last paragraph."""
+        p = self.qkv(x, out_dtype=self.dtype)                      # [q | k | v | a gate a head]
+        C = self.nq * self.d + self.nkv * (self.d + self.dv)
+        slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
+        vt = self.dtype == torch.bfloat16
+        tails = None
+        if self.taps > 1:
+            tails = cache.states.get("conv_tail")
+            if tails is None:
+                raise RuntimeError("an attention with a convolution was given no state slots")
+        q = kernels.conv_qkv_rows(p, self.conv_w, tails, ctx.state_slots, ctx.tok_seq, ctx.cu_q, self.q_norm_w, self.k_norm_w,
+                                  self.qk_norm_eps, slots, cache.k, cache.v, self.nq, self.nkv, self.d, self.dv, v_grouped=vt,
+                                  value_unit_norm=self.value_unit, talk=self.talk)
+        if self.taps > 1 and cache.write:
+            kernels.conv_tail(p[:, :C], tails, ctx.state_slots, ctx.cu_q)
+        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt)
+        if self.head_gate:
+            kernels.head_gate_(a, p[:, C:], self.nq)
+        return self.o(a, out_dtype=self.dtype, allow_split=True)

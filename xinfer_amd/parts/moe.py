@@ -10,7 +10,10 @@ device and the experts' kernels find their rows from it, so decode steps can be 
 Options, each a parameter of the spec: `gated: False` makes an expert down(act(up x)) with the up rows
 alone ([E, F, H]) and takes the activations without a gate as well ("relu2": the square of relu);
 `scores: "all"` weighs the chosen experts by their softmax scores over ALL experts, divided by the
-chosen ones' sum + 1e-20 (in place of the softmax over the chosen logits); `shared` = {intermediate_size,
+chosen ones' sum + 1e-20 (in place of the softmax over the chosen logits), `scores: "sigmoid"` by sigmoid(z) of each
+chosen expert as it is (nothing is divided; the largest logits are the largest scores); `weigh: "input"` lets the
+weight multiply what the expert SEES, sum of expert_e(weight_e * x), instead of what it returns (the experts' first
+products are linear, so the kernels put the weight on their float32 sums, before the activation); `shared` = {intermediate_size,
 activation, gated, gate}: one more expert of the same form that every token takes, added to the result,
 times sigmoid(w_g . x) with a vector w_g of its own if `gate` says so (that product rides with the
 router's, in float32).
@@ -52,6 +55,12 @@ class RoutedExperts(FeedForward):
         self.gated = bool(spec.get("gated", True))
         self._check_act(self.activation, self.gated)
         self.all_scores = self._scores(spec) == "all"
+        self.sigmoid_scores = self._scores(spec) == "sigmoid"
+        self.weigh_input = str(spec.get("weigh", "output")) == "input"
+        if str(spec.get("weigh", "output")) not in ("input", "output"):
+            raise ValueError(f"weigh {spec.get('weigh')!r}: 'output' (the expert's result) or 'input'")
+        if self.weigh_input and not self.gated:
+            raise NotImplementedError("a weight on the experts' input is built for gated experts")
         if not (0 < self.top <= self.experts):
             raise ValueError(f"{self.top} of {self.experts} experts cannot be chosen")
         sh = spec.get("shared")
@@ -76,8 +85,8 @@ class RoutedExperts(FeedForward):
     @staticmethod
     def _scores(spec: PartSpec) -> str:
         scores = str(spec.get("scores", "chosen"))
-        if scores not in ("chosen", "all"):
-            raise ValueError(f"router scores {scores!r}: 'chosen' (softmax over the chosen logits) or 'all'")
+        if scores not in ("chosen", "all", "sigmoid"):
+            raise ValueError(f"router scores {scores!r}: 'chosen' (softmax over the chosen logits), 'all' or 'sigmoid'")
         return scores
 
     @classmethod
@@ -134,15 +143,17 @@ class RoutedExperts(FeedForward):
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         opens = bool(self.shared and self.shared["open"])
         routed = kernels.moe_route(x, self.router_w, self.router_b, self.top, all_scores=self.all_scores,
-                                   extra_rows=1 if opens else 0)
+                                   extra_rows=1 if opens else 0, sigmoid=self.sigmoid_scores)
         idx, wt = routed[0], routed[1]
         # a step that brings portions is never recorded: with many rows an expert it may read the experts' row
         # counts on the host and hand each expert's rows to the vendor library, as the dense products of many rows go
         if (ctx.max_q_len > 1 and x.dtype == torch.bfloat16 and self.LIBRARY
                 and x.shape[0] * self.top >= kernels.MOE_LIBRARY_ROWS * self.experts):
-            out = kernels.moe_experts_library(x, self.gate_up, self.down, idx, wt, self.activation, gated=self.gated)
+            out = kernels.moe_experts_library(x, self.gate_up, self.down, idx, wt, self.activation, gated=self.gated,
+                                              weigh_input=self.weigh_input)
         else:
-            out = kernels.moe_experts(x, self.gate_up, self.down, idx, wt, self.activation, gated=self.gated)
+            out = kernels.moe_experts(x, self.gate_up, self.down, idx, wt, self.activation, gated=self.gated,
+                                      weigh_input=self.weigh_input)
         if self.shared:
             out = self._add_shared(out, x, routed[2][:, 0] if opens else None)
         return out
