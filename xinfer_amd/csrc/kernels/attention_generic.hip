@@ -26,8 +26,9 @@
 
 namespace xi {
 
-constexpr int kMaxHeadDim = 256;       // heads up to this size take the first instantiation,
+constexpr int kMaxHeadDim = 256;       // value heads up to this size take the first instantiation,
 constexpr int kMaxHeadDimWide = 640;   // up to this the second
+constexpr int kMaxKeyDim = 8192;       // key heads: the query sits in LDS, as long as it is
 constexpr int kAttnWaves = 4;
 
 template <typename T, int MAXD>
@@ -37,7 +38,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const int* __restrict__ positions, T* __restrict__ out, float scale, int window, int page_size,
     int nq, int nkv, int d, int dv, int v_grouped, float softcap, const float* __restrict__ slopes,
     const float* __restrict__ sinks, int values_in_keys, int nkk) {
-  __shared__ float q_s[MAXD];
+  extern __shared__ float q_s[];       // [d]
   __shared__ float acc_s[kAttnWaves][MAXD];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
 
@@ -157,7 +158,7 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
            "attention: bad sizes T=%d nq=%d nkv=%d page=%d max_pages=%d", n_tok, nq, nkv, page_size, max_pages);
   XI_CHECK(nq % nkv == 0, "attention: %d query heads are not a multiple of %d kv heads", nq, nkv);
   XI_CHECK(nkk > 0 && nq % nkk == 0 && (!values_in_keys || nkk == nkv), "attention: %d query heads on %d key heads", nq, nkk);
-  XI_CHECK(d > 0 && d <= kMaxHeadDimWide, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDimWide);
+  XI_CHECK(d > 0 && d <= kMaxKeyDim, "attention: head_dim %d is outside 1..%d", d, kMaxKeyDim);
   XI_CHECK(dv > 0 && dv <= kMaxHeadDimWide, "attention: value head size %d is outside 1..%d", dv, kMaxHeadDimWide);
   XI_CHECK(!values_in_keys || (dv <= d && !v_grouped), "attention: values that are the keys' first dims need dv <= d");
   XI_CHECK(softcap >= 0.f, "attention: the soft cap must be positive (0: none), got %g", (double)softcap);
@@ -165,9 +166,10 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
   XI_CHECK(!v_grouped || page_size % 8 == 0, "attention: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d", page_size);
   if (n_tok == 0) return 0;
   dim3 grid(n_tok, nq);
-  const bool wide = d > kMaxHeadDim || dv > kMaxHeadDim;
+  const bool wide = dv > kMaxHeadDim;
+  const size_t q_bytes = (size_t)d * sizeof(float);
 #define XI_AG(TT, MAXD)                                                                                                 \
-  attention_generic_kernel<TT, MAXD><<<grid, kAttnWaves * kWave, 0, stream>>>(                                          \
+  attention_generic_kernel<TT, MAXD><<<grid, kAttnWaves * kWave, q_bytes, stream>>>(                                          \
       (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, block_tables, max_pages, tok_seq, positions, (TT*)out, scale, \
       window, page_size, nq, nkv, d, dv, v_grouped, softcap, slopes, sinks, values_in_keys, nkk)
   if (dtype == kF32 && !wide) XI_AG(float, kMaxHeadDim);
