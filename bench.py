@@ -42,6 +42,10 @@ is, Mufenex with routed experts and no window, at equal sizes.
 `--design debusun[:SIZE]` times the Debusun family (layers of attention over a latent with sinks and a gate, of
 windowed attention whose heads are normed after the rotation, and of a selective state space, in turn; dense
 feed-forwards of a squared relu; a table of token pairs beside the embedding) beside dense Mufenex at equal sizes.
+`--design vuzazen[:SIZE]` times the Vuzazen family (layers of attention over a latent with the queries through a latent
+of their own, of a matrix memory, and of attention behind a short convolution whose heads' scores are mixed, in turn;
+dense silu feed-forwards, or experts that see the token times its score) beside Debusun at equal sizes, which has no
+experts: at the size with experts its feed-forwards are dense of the same active width.
 """
 from __future__ import annotations
 
@@ -86,6 +90,10 @@ DESIGN_SIZES = {
     "4k-moe": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, ff=12288, window=2048, experts=8, top=2),
     "2k-v": dict(width=2048, heads=16, kv_heads=4, dim=64, vdim=128, ff=8192, window=512, experts=16, top=2),
     "1k-moe": dict(width=1024, heads=16, kv_heads=8, dim=128, vdim=128, ff=3072, window=1024, experts=8, top=2),
+    # two kv heads: the heads' mix scores a query against both kv heads' dims at once (256 of them)
+    "1k-g2": dict(width=1024, heads=16, kv_heads=2, dim=128, vdim=128, ff=3072, window=1024, experts=0, top=0),
+    "4k-g2": dict(width=4096, heads=32, kv_heads=2, dim=128, vdim=128, ff=12288, window=2048, experts=0, top=0),
+    "4k-g2-moe": dict(width=4096, heads=32, kv_heads=2, dim=128, vdim=128, ff=12288, window=2048, experts=8, top=2),
 }
 LILALORN_SIZES = ("1k-moe", "4k-moe", "2k-v")      # the sizes with experts: every Lilalorn layer has them
 DEBUSUN_SIZES = ("1k", "4k")                        # the dense sizes: every Debusun feed-forward is dense
@@ -93,8 +101,13 @@ DEBUSUN_SIZES = ("1k", "4k")                        # the dense sizes: every Deb
 # one head), the state space's head and state sizes (its inner width is twice the model's)
 DEBUSUN_LATENT = dict(kv_rank=192, rot_dim=64)
 DEBUSUN_STATE = dict(vdim=64, state=128, groups=1, conv=4, norm_groups=1)
-DESIGN_CHOICES = {"mufenex": (tuple(DESIGN_SIZES), "qwen3"), "lilalorn": (LILALORN_SIZES, "mufenex"),
-                  "debusun": (DEBUSUN_SIZES, "mufenex")}
+VUZAZEN_SIZES = ("1k-g2", "4k-g2", "4k-g2-moe")
+# Vuzazen's own sizes at every width: the latents (keys as Debusun's; queries through 3/8 of the width), the memories'
+# heads (a quarter as many as the query heads, keys as wide as the attention's and values twice that), the taps
+VUZAZEN_LATENT = dict(kv_rank=192, rot_dim=64)
+VUZAZEN_TAPS = 4
+DESIGN_CHOICES = {"mufenex": (tuple(k for k in DESIGN_SIZES if "g2" not in k), "qwen3"), "lilalorn": (LILALORN_SIZES, "mufenex"),
+                  "debusun": (DEBUSUN_SIZES, "mufenex"), "vuzazen": (VUZAZEN_SIZES, "debusun")}
 DESIGN_VOCAB = 32000
 MODELS = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 CONTEXT = 4096
@@ -232,8 +245,8 @@ def product(spec: str, dev="cuda:0") -> int:
 
 def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, context: int, prefill_tokens: int,
                    family: str = "both", only: str = "all") -> int:
-    """Mufenex beside Qwen3, or Lilalorn or Debusun beside Mufenex, at equal sizes: ms of the prefill of one prompt
-    and of a decode step."""
+    """Mufenex beside Qwen3, Lilalorn or Debusun beside Mufenex, or Vuzazen beside Debusun, at equal sizes: ms of the
+    prefill of one prompt and of a decode step."""
     import torch
     from xinfer_amd.engine import ModelRunner, StepEntry, build_model
     from xinfer_amd.models import config_from_dict
@@ -268,7 +281,7 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
                      vocab_size=DESIGN_VOCAB, sliding_window=z["window"], max_position_embeddings=2 * context)
         if name == "mufenex":
             return {"mufenex": mufenex, "qwen3": qwen3}
-        if name == "debusun":
+        if name in ("debusun", "vuzazen"):
             # layers of a latent, windowed attention, a state space and windowed attention again, in turn; all of them
             # are one span that runs once, so that the start of a pass is in the step
             rot = dict(dims=z["dim"], base=500000.0)
@@ -285,7 +298,20 @@ def design_compare(spec: str, layers, steps: int, warmup: int, batch: int, conte
                        "max_positions": 2 * context, "loop": {"start": 0, "stop": layers, "times": 1},
                        "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": z["ff"]}}
                                   for i in range(layers)]}
-            return {"debusun": debusun, "mufenex": mufenex}
+            if name == "debusun":
+                return {"debusun": debusun, "mufenex": mufenex}
+            # Vuzazen: a latent, a memory, attention behind a convolution with mixed heads, a memory, in turn; no windows
+            vlat = dict(heads=z["heads"], dim=z["dim"], vdim=z["vdim"], q_rank=3 * z["width"] // 8,
+                        scale=(z["dim"] + VUZAZEN_LATENT["rot_dim"]) ** -0.5, **VUZAZEN_LATENT,
+                        rot=dict(dims=VUZAZEN_LATENT["rot_dim"], base=500000.0))
+            vatt = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5, conv=VUZAZEN_TAPS)
+            mem = dict(heads=max(1, z["heads"] // 4), dim=z["dim"], vdim=2 * z["dim"], gate_cap=15.0)
+            vkinds = [("latent_attention", vlat), ("mlstm", mem), ("attention", vatt), ("mlstm", mem)]
+            vuzazen = {"architecture": "Vuzazen", "vocab": DESIGN_VOCAB, "width": z["width"], "norm": {"eps": 1e-6},
+                       "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 31}},
+                       "max_positions": 2 * context,
+                       "layers": [{"type": vkinds[i % 4][0], "mixer": vkinds[i % 4][1], "mlp": mlp} for i in range(layers)]}
+            return {"vuzazen": vuzazen, "debusun": debusun}
         # Lilalorn: layers of attention beside retention and of gated linear attention in turn; the states' heads are a
         # quarter as many as the query heads, keys as wide as the attention's and values twice that
         mixer.pop("mask")
@@ -432,7 +458,7 @@ def main() -> int:
                     help="serving workloads: read every step's tokens on the host before the next step is planned")
     ap.add_argument("--product", default=None, metavar="M,N,K[,slices[,shape]]",
                     help="time one bfloat16 product alone in the many-row tiled kernel and in the vendor library")
-    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]|debusun[:SIZE]",
+    ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]|debusun[:SIZE]|vuzazen[:SIZE]",
                     help="time another model family beside its closest one (Mufenex beside Qwen3, Lilalorn or Debusun beside Mufenex) at equal sizes (a line of its own; --layers, --steps, "
                          "--warmup, --batch, --context, --prefill-tokens and --only apply)")
     ap.add_argument("--family", choices=["both", "debusun", "lilalorn", "mufenex", "qwen3"], default="both",

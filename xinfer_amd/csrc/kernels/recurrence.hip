@@ -14,8 +14,10 @@
 //              are float32.
 //   gates      a_t[i] = gates[t, h, 0] for every channel and the value row times gates[t, h, 1], both made
 //              beforehand (float32 [T, H, 2]: the keep and take factors of a matrix memory, mlstm.hip).
-// With `v_cols` < dv the value rows hold v_cols columns a head and the state's further columns read the value 1:
-// column v_cols of the state is then the sum of the (decayed, weighted) keys alone, the normalizer of a matrix memory.
+// With `v_cols` = dv - 1 the value rows hold v_cols columns a head and the state's last column reads the value 1: it
+// is then the sum n of the (decayed, weighted) keys alone, the normalizer of a matrix memory, and its result n . q.
+// That column is no lane's: thread c keeps n[c] in a register beside the channel it fetches, and the workgroup adds up
+// n[c] q[c] once a token (the grid covers the v_cols columns; the first tile's workgroup writes the column).
 // With `group_heads` g > 1, q and k have one set of dk columns for every g heads (head h reads set h / g).
 // q, k and v are columns of a packed projection (a row stride and a column offset each); q and k are
 // multiplied by `q_scale` / `k_scale` in float32 as they are read.
@@ -67,11 +69,13 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     int H, int dk, int dv, float q_scale, float k_scale) {
   __shared__ __attribute__((aligned(16))) float qs[2][kScanWaves * 64], ks[2][kScanWaves * 64], as[2][kScanWaves * 64];
   __shared__ float part[2][kScanWaves][kScanCols];
+  __shared__ float npart[2][kScanWaves];
   const int b = blockIdx.x, h = blockIdx.y, j = blockIdx.z * kScanCols + (threadIdx.x & 63);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t0 = first[b], t1 = last[b];
   if (t1 <= t0) return;
-  const bool col = j < dv;
+  const bool ones = v_cols < dv;            // the state's last column is the keys' own sum
+  const bool col = j < v_cols;
   const long long from = in_idx ? in_idx[b] : -1, to = out_idx ? out_idx[b] : -1;      // negative: from zeros / kept nowhere
   const float* S = state_in + (size_t)(from < 0 ? 0 : from) * in_stride + (size_t)h * dk * dv;
   float s[RPT];
@@ -82,6 +86,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
   }
   float all_decays = 1.f;               // of channel c, over the item's tokens
   const int c = threadIdx.x;            // the channel this thread fetches for the workgroup
+  float nc = (ones && from >= 0 && c < dk) ? S[(size_t)c * dv + v_cols] : 0.f;
   const float hd = head_decay ? head_decay[h] : 0.f;
   const float zb = (z_bias && c < dk) ? z_bias[h * dk + c] : 0.f;
   const int qk0 = (h / group_heads) * dk;       // the head's set of q and k columns
@@ -117,6 +122,11 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     all_decays *= fa;
     const float a_now = fa;
     const float vj = v_next;
+    if (ones) {                          // (this token's k and q are in LDS since the last barrier)
+      nc = fmaf(a_now, nc, dt * ks[cur][c]);
+      const float nq = wave_sum(nc * qs[cur][c]);
+      if (out && lane == 0) npart[cur][wave] = nq;
+    }
     if (t + 1 < t1) {
       dt = step_of(t + 1);
       fetch(t + 1, dt, fq, fk, fa);
@@ -148,6 +158,8 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
     __syncthreads();
     if (out && wave == 0 && col)
       out[((size_t)t * H + h) * dv + j] = (part[cur][0][lane] + part[cur][1][lane]) + (part[cur][2][lane] + part[cur][3][lane]);
+    if (out && ones && blockIdx.z == 0 && threadIdx.x == 0)
+      out[((size_t)t * H + h) * dv + v_cols] = (npart[cur][0] + npart[cur][1]) + (npart[cur][2] + npart[cur][3]);
   }
   if (to >= 0) {
     float* D = state_out + (size_t)to * out_stride + (size_t)h * dk * dv;
@@ -156,6 +168,7 @@ __global__ __launch_bounds__(kScanWaves* kWave) void linear_scan_kernel(
       const int i = wave * RPT + r;
       if (col && i < dk) D[(size_t)i * dv + j] = s[r];
     }
+    if (ones && blockIdx.z == 0 && c < dk) D[(size_t)c * dv + v_cols] = nc;
   }
   if (decay_out && blockIdx.z == 0 && c < dk) decay_out[((size_t)b * H + h) * dk + c] = all_decays;
 }
@@ -231,7 +244,7 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
   XI_CHECK(dk <= kScanWaves * 64, "linear_scan: key heads of up to %d channels, not %d", kScanWaves * 64, dk);
   XI_CHECK((z != nullptr) + (head_decay != nullptr) + (step != nullptr) + (gates != nullptr) == 1,
            "linear_scan: a decay per token and channel, per head, per token and head from a step size, or ready-made gates: one of them");
-  XI_CHECK(v_cols > 0 && v_cols <= dv, "linear_scan: %d value columns in rows for a state of %d", v_cols, dv);
+  XI_CHECK(v_cols > 0 && (v_cols == dv || v_cols == dv - 1), "linear_scan: %d value columns in rows for a state of %d", v_cols, dv);
   XI_CHECK(step == nullptr || (step_bias && decay_log && step_stride >= H), "linear_scan: a step size needs its bias and its rate");
   XI_CHECK(group_heads >= 1 && H % group_heads == 0, "linear_scan: %d heads in groups of %d", H, group_heads);
   XI_CHECK(z == nullptr || tau > 0.f, "linear_scan: tau must be positive");
@@ -240,7 +253,7 @@ int xi_linear_scan(const void* q, long long q_stride, const void* k, long long k
            "linear_scan: states need a place of at least H dk dv floats each");
   XI_CHECK(first && last, "linear_scan: the items' token ranges are missing");
   if (n_items == 0) return 0;
-  dim3 grid((unsigned)n_items, (unsigned)H, (unsigned)((dv + kScanCols - 1) / kScanCols));
+  dim3 grid((unsigned)n_items, (unsigned)H, (unsigned)((v_cols + kScanCols - 1) / kScanCols));
   XI_CHECK(grid.y <= 65535u && grid.z <= 65535u, "linear_scan: too many heads or value columns");
   const float inv_tau = z ? 1.f / tau : 0.f;
   const int rpt = (dk + kScanWaves - 1) / kScanWaves;

@@ -303,8 +303,8 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     or `step` [T, H] (columns of a projection, in q's type), `step_bias` and `decay_log` float32 [H]: the step size d =
     softplus(step + step_bias), a = exp(-exp(decay_log) d) per token and head, and the token's value row times d.
     Or `gates` float32 [T, H, 2], made beforehand: a = gates[t, h, 0] and the token's value row times gates[t, h, 1].
-    `value_cols` c < value_dim: v is [T, H c] and the state's columns from c on read the value 1 (column c then holds
-    the decayed sum of the weighted keys alone).
+    `value_cols` = value_dim - 1: v is [T, H (value_dim - 1)] and the state's last column reads the value 1 (it then
+    holds the decayed sum of the weighted keys alone, and the results' last column that sum times q).
     `groups` G: q and k are [T, G dk] and head h reads the columns of group h // (H / G).
     state float32 [slots, H, dk, dv] (slots may be strided); state_slots int64 [B]; cu_q int32 [B + 1].
     Returns o float32 [T, H, dv].
@@ -319,7 +319,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.
     if G <= 0 or H % G:
         raise KernelError(f"linear_scan: {H} heads in {G} groups")
     vc = dv if value_cols is None else int(value_cols)
-    if not (0 < vc <= dv):
+    if vc not in (dv, dv - 1) or vc <= 0:
         raise KernelError(f"linear_scan: {vc} value columns for a state of {dv}")
     qs, ks, vs = _columns(q, G * dk, "linear_scan: q"), _columns(k, G * dk, "linear_scan: k"), _columns(v, H * vc, "linear_scan: v")
     if k.shape[0] != T or v.shape[0] != T or q.dtype != k.dtype or q.dtype != v.dtype or not (q.device == k.device == v.device):
