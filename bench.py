@@ -461,7 +461,7 @@ def main() -> int:
     ap.add_argument("--design", default=None, metavar="mufenex[:SIZE]|lilalorn[:SIZE]|debusun[:SIZE]|vuzazen[:SIZE]",
                     help="time another model family beside its closest one (Mufenex beside Qwen3, Lilalorn or Debusun beside Mufenex) at equal sizes (a line of its own; --layers, --steps, "
                          "--warmup, --batch, --context, --prefill-tokens and --only apply)")
-    ap.add_argument("--family", choices=["both", "debusun", "lilalorn", "mufenex", "qwen3"], default="both",
+    ap.add_argument("--family", choices=["both", "debusun", "lilalorn", "mufenex", "qwen3", "vuzazen"], default="both",
                     help="--design: time one of the two families only (for profiling)")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "

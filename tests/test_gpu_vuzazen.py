@@ -329,6 +329,8 @@ MIXED_CASES = [  # H, G, d, dv, scale, L, page
     (3, 1, 12, 20, 0.5, 150, 8),
     (4, 2, 128, 64, 0.09, 400, 64),
     (6, 3, 32, 128, 0.18, 200, 32),
+    (24, 2, 64, 128, 0.12, 130, 16),          # twelve heads a group: a group's rows in one block, or in two
+    (40, 2, 32, 64, 0.2, 100, 16),            # twenty heads a group
     (4, 4, 64, 64, 0.12, 200, 64),
     (12, 12, 64, 32, 0.12, 100, 16),          # a key head of 768 dims: the generic kernel alone
 ]
@@ -354,6 +356,12 @@ def _mixed_case(case, dtype, matrix_cores, tail=9):
     k_pool, v_pool, table = k_pool.to(DEV), v_pool.to(DEV), table.to(DEV)
     qf = kernels.conv_qkv_rows(packed, None, None, _i64([0]), _i32([0] * L), _i32([0, L]), None, None, 1e-5, slots.to(DEV), k_pool,
                                v_pool, H, G, d, dv, v_grouped=grouped, value_unit_norm=False, talk=talk.to(DEV))
+    if dtype == "bfloat16":
+        # what the attention kernels are held to: the scores of the mixed queries as they were rounded (the mix itself
+        # is held to the plain one where the rows are tested; planted scores of 30 make its rounding show in the weights)
+        mixed = torch.einsum("ihx,jx->hij", qf.cpu().double(), k.double().reshape(L, G * d)) * scale
+        assert (mixed - scores).abs().max() < 0.02 * scores.abs().max()
+        want = torch.stack([plain.causal_softmax(mixed[h]) @ v.double()[:, h // (H // G)] for h in range(H)], dim=1).reshape(L, H * dv)
 
     def run(positions):
         qs = qf[positions[0]:positions[-1] + 1]
@@ -361,6 +369,14 @@ def _mixed_case(case, dtype, matrix_cores, tail=9):
         if not matrix_cores:
             return kernels.attention_generic(qs, k_pool, v_pool, table, torch.zeros_like(pos), pos, scale, 0, v_grouped=grouped)
         n, ctx = len(positions), positions[-1] + 1
+        per = H // G
+        if n == 1 and per >= 4:                     # a group's heads as the rows of blocks that read the one key head
+            shape = 1 if kernels.attention_biased_block(G * d, dv, 1, 1) >= per else 0
+            rows_ = kernels.attention_biased_block(G * d, dv, 1, shape)
+            tiles = _i32([[0, c * per + b * rows_] for c in range(G) for b in range(-(-per // rows_))])
+            out = kernels.attention_biased_bf16(qs.reshape(H, 1, G * d), k_pool, v_pool, table, tiles, _i32([0, H]), _i32([ctx]), scale, 0,
+                                                small=shape, split_keys=64 if positions[0] % 2 else 0, span=ctx, rows_heads=H)
+            return out.view(1, H * dv)
         rows, shape = kernels.prefill_tiles([n], [ctx], G * d, H, G, block_of=lambda s_: kernels.attention_biased_block(G * d, dv, H // G, s_))
         tiles = torch.tensor(rows, dtype=torch.int32, device=DEV).reshape(-1, 2)
         split, span = (64, ctx) if n == 1 and positions[0] % 2 else (0, 0)     # every other single token in slices of 64 keys

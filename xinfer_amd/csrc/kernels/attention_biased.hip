@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale,
     float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks, int window, int page_shift, int nq,
     int nkv, int d, int dv, float* __restrict__ part_o, float* __restrict__ part_ml, int split_keys, int max_splits,
-    int rows_heads, int nkk) {
+    int rows_heads, int nkk, int rows_kv) {
   const int page = 1 << page_shift;
   constexpr int NT = 64 * NWV;                    // threads
   constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
@@ -69,8 +69,17 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
   const int h0 = kvh * g + (blockIdx.x - kvh * groups) * GH;
   const int kh = kvh / (nkv / nkk);               // the kv head's key head
   const int seq = tiles[2 * blockIdx.y], q0_blk = tiles[2 * blockIdx.y + 1];
-  const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
+  const int q_begin = cu_q[seq], q_rows = cu_q[seq + 1] - q_begin;
   const int ctx = ctx_lens[seq];
+  // rows_heads with rows_kv > 1: the rows are heads that share the one key head and read rows_kv value heads, rows_heads
+  // / rows_kv rows each; a block's rows lie within one value head's rows (the host cuts the blocks so)
+  int v_heads = nkv, v_head = kvh, q_len = q_rows;
+  if (rows_heads > 0 && rows_kv > 1) {
+    const int per = rows_heads / rows_kv;
+    v_heads = rows_kv;
+    v_head = q0_blk / per;
+    q_len = min(q_rows, (v_head + 1) * per);
+  }
   // rows_heads > 0: the sequence's rows are the query heads of its one new token (all of them read the one kv head:
   // attention over a latent), so every row stands at the last position and row i has sink i
   const int step = rows_heads > 0 ? 0 : 1;
@@ -191,7 +200,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_biased_lds_kernel(
       int key0 = kb + 8 * c_vkg[i];
       key0 = key0 > k_last ? (k_last & ~7) : key0;
       const int vp = bt_s[key0 >> page_shift];
-      vreg[i] = ld8(vt_cache + ((size_t)vp * nkv + kvh) * v_head_stride +
+      vreg[i] = ld8(vt_cache + ((size_t)vp * v_heads + v_head) * v_head_stride +
                     ((size_t)((key0 & (page - 1)) >> 3) * dv + c_vrow[i]) * 8);     // [offset / 8, dv, 8]
     }
   };
@@ -460,12 +469,16 @@ int xi_attention_biased_block(int d, int dv, int g, int small) {
 
 // tiles int32 [n_tiles, 2] = (sequence, first query position of the block within the sequence's portion).
 // q [T, nq, d]; K pool [pages, nkv, page, d]; V pool [pages, nkv, page / 8, dv, 8]; out [T, nq * dv].
+// rows_heads H > 0 (nq = nkv = 1): the rows of a sequence are the H heads of its one token; rows_kv G > 1: the V pool has
+// G heads, rows h H / G .. (h + 1) H / G - 1 read value head h, and no block of `tiles` crosses such a border.
 // softcap 0: none; slopes null: none; sinks null: none, else float32 [nq], exp(sinks[h]) joins head h's denominator.
 int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
                              int max_pages, const int* tiles, int n_tiles, const int* cu_q, const int* ctx_lens,
                              void* out, float scale, float softcap, const float* slopes, const float* sinks, int window,
                              int page, int nq, int nkv, int d, int dv, int small, float* part_o, float* part_ml, int split_keys,
-                             int max_splits, int n_tok, int rows_heads, int nkk, hipStream_t stream) {
+                             int max_splits, int n_tok, int rows_heads, int nkk, int rows_kv, hipStream_t stream) {
+  XI_CHECK(rows_kv >= 1 && (rows_kv == 1 || (rows_heads > 0 && rows_heads % rows_kv == 0)),
+           "attention_biased: %d value heads for rows that are %d heads", rows_kv, rows_heads);
   XI_CHECK(nkk > 0 && nkv % nkk == 0, "attention_biased: %d kv heads on %d key heads", nkv, nkk);
   XI_CHECK(rows_heads == 0 || (rows_heads > 0 && nq == 1 && nkv == 1 && slopes == nullptr && n_tok % rows_heads == 0),
            "attention_biased: rows that are the %d heads of a token come with one head, no slopes and whole tokens", rows_heads);
@@ -502,7 +515,7 @@ int xi_attention_biased_bf16(const void* q, const void* k_cache, const void* vt_
     kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
                                           block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
                                           scale, softcap, slopes, sinks, window, page_shift, nq, nkv, d,\
-                                          dv, part_o, part_ml, split_keys, max_splits, rows_heads, nkk);\
+                                          dv, part_o, part_ml, split_keys, max_splits, rows_heads, nkk, rows_kv);\
   } while (0)
 #define XI_PB_GH(KC, DT, NQT, NWV)             \
   do {                                         \

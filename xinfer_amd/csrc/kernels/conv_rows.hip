@@ -24,7 +24,29 @@
 
 namespace xi {
 
-constexpr int kRowThreads = 256;
+constexpr int kRowThreads = 1024;   // a token's row is a few thousand channels: every thread a few, all loads in flight at once
+constexpr int kTapsUnrolled = 8;    // convolutions of up to this many taps ask for all their inputs before the first sum
+
+template <typename T>
+__device__ __forceinline__ void store_run8(T* dst, const float (&v)[8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) dst[i] = from_float<T>(v[i]);
+}
+template <>
+__device__ __forceinline__ void store_run8<bf16>(bf16* dst, const float (&v)[8]) {      // 16 bytes where the place allows it
+  if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    unsigned u[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bf16 lo = __float2bfloat16(v[2 * i]), hi = __float2bfloat16(v[2 * i + 1]);
+      u[i] = (unsigned)*reinterpret_cast<const unsigned short*>(&lo) | ((unsigned)*reinterpret_cast<const unsigned short*>(&hi) << 16);
+    }
+    *reinterpret_cast<uint4*>(dst) = make_uint4(u[0], u[1], u[2], u[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = __float2bfloat16(v[i]);
+  }
+}
 
 template <typename T>
 __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
@@ -33,12 +55,33 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
     const int* __restrict__ cu_q, const float* __restrict__ qw, const float* __restrict__ kw, float eps, int v_unit,
     const float* __restrict__ talk, const long long* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ k_cache,
     T* __restrict__ v_cache, int page_size, int nq, int nkv, int d, int dv, int v_grouped) {
-  extern __shared__ float row[];                 // the token's C channels after the convolution
+  extern __shared__ float row[];                 // the token's C channels after the convolution, then the heads' mix
   __shared__ float scratch[kRowThreads / kWave];
   const int t = blockIdx.x;
   const int nqd = nq * d, nkd = nkv * d, nvd = nkv * dv, C = nqd + nkd + nvd;
+  float* talk_s = row + C;                       // [nq, nq]
+  if (talk)
+    for (int i = threadIdx.x; i < nq * nq; i += kRowThreads) talk_s[i] = talk[i];
   const T* ur = u + (size_t)t * u_stride;
-  if (taps > 1) {
+  if (taps > 1 && taps <= kTapsUnrolled) {
+    const int b = tok_seq[t];
+    const int t0 = cu_q[b];
+    const float* tail = tails + (size_t)state_slots[b] * tail_stride;
+    for (int c = threadIdx.x; c < C; c += kRowThreads) {
+      float x[kTapsUnrolled], w[kTapsUnrolled];
+#pragma unroll
+      for (int j = 0; j < kTapsUnrolled; ++j) {
+        const int s = t - (taps - 1) + j;
+        x[j] = j >= taps ? 0.f : s >= t0 ? to_float(u[(size_t)s * u_stride + c]) : tail[(size_t)(taps - 1 - (t0 - s)) * C + c];
+        w[j] = j < taps ? cw[(size_t)c * taps + j] : 0.f;
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < kTapsUnrolled; ++j)
+        if (j < taps) acc = fmaf(w[j], x[j], acc);
+      row[c] = acc;
+    }
+  } else if (taps > 1) {
     const int b = tok_seq[t];
     const int t0 = cu_q[b];
     const float* tail = tails + (size_t)state_slots[b] * tail_stride;
@@ -77,14 +120,29 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
     }
   }
   __syncthreads();
-  if (talk) {
+  if (talk && d % 8 == 0) {                      // eight dims of one (head, kv head) a thread
     const int g = nq / nkv;                      // query heads on a kv head
+    T* qo = q_out + (size_t)t * nq * nkd;
+    for (int i = threadIdx.x; i < nq * nkd / 8; i += kRowThreads) {
+      const int h = (8 * i) / nkd, r = 8 * i - h * nkd;
+      const int c = r / d, e = r - c * d;
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < g; ++j) {
+        const float w = talk_s[h * nq + c * g + j];
+        const float* src = row + (c * g + j) * d + e;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) acc[x] = fmaf(w, src[x], acc[x]);
+      }
+      store_run8<T>(qo + 8 * i, acc);
+    }
+  } else if (talk) {
+    const int g = nq / nkv;
     T* qo = q_out + (size_t)t * nq * nkd;
     for (int i = threadIdx.x; i < nq * nkd; i += kRowThreads) {
       const int h = i / nkd, r = i - h * nkd;
       const int c = r / d, e = r - c * d;
       float acc = 0.f;
-      for (int j = 0; j < g; ++j) acc = fmaf(talk[h * nq + c * g + j], row[(c * g + j) * d + e], acc);
+      for (int j = 0; j < g; ++j) acc = fmaf(talk_s[h * nq + c * g + j], row[(c * g + j) * d + e], acc);
       qo[i] = from_float<T>(acc);
     }
   } else {
@@ -122,22 +180,21 @@ __global__ __launch_bounds__(256) void head_gate_kernel(T* __restrict__ x, const
   x[i] = from_float<T>(to_float(x[i]) * (1.f / (1.f + expf(-gv))));
 }
 
-// one wave a row
+// a workgroup a row
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void rows_rmsnorm_kernel(const TI* __restrict__ x, long long x_stride,
                                                            const float* __restrict__ w, float eps, TO* __restrict__ out,
                                                            int n_rows, int n) {
-  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= n_rows) return;
-  const int lane = threadIdx.x & 63;
+  __shared__ float scratch[4];
+  const int r = blockIdx.x;
   const TI* xr = x + (size_t)r * x_stride;
   float ss = 0.f;
-  for (int i = lane; i < n; i += kWave) {
+  for (int i = threadIdx.x; i < n; i += 256) {
     const float v = to_float(xr[i]);
     ss = fmaf(v, v, ss);
   }
-  const float inv = rsqrtf(wave_sum(ss) / (float)n + eps);
-  for (int i = lane; i < n; i += kWave) out[(size_t)r * n + i] = from_float<TO>(to_float(xr[i]) * inv * (w ? w[i] : 1.f));
+  const float inv = rsqrtf(block_sum<4>(ss, scratch) / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += 256) out[(size_t)r * n + i] = from_float<TO>(to_float(xr[i]) * inv * (w ? w[i] : 1.f));
 }
 
 }  // namespace xi
@@ -164,8 +221,8 @@ int xi_conv_qkv_rows(const void* u, long long u_stride, int dtype, const float* 
            "conv_qkv_rows: a convolution of %d taps needs its weights and the requests' tails", taps);
   XI_CHECK(!v_grouped || page_size % 8 == 0, "conv_qkv_rows: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d",
            page_size);
-  const size_t lds = (size_t)C * sizeof(float);
-  XI_CHECK(lds <= 150 * 1024, "conv_qkv_rows: a row of %lld channels does not fit in LDS", C);
+  const size_t lds = ((size_t)C + (talk ? (size_t)nq * nq : 0)) * sizeof(float);
+  XI_CHECK(lds <= 150 * 1024, "conv_qkv_rows: a row of %lld channels (and %d heads' mix) does not fit in LDS", C, nq);
   if (n_tok == 0) return 0;
 #define XI_CR(TT)                                                                                                     \
   do {                                                                                                                \
@@ -205,7 +262,7 @@ int xi_rows_rmsnorm(const void* x, long long x_stride, int in_dtype, const float
                     int n_rows, int n, hipStream_t stream) {
   XI_CHECK(n_rows >= 0 && n > 0 && x_stride >= n, "rows_rmsnorm: bad sizes rows=%d n=%d", n_rows, n);
   if (n_rows == 0) return 0;
-  const unsigned blocks = (unsigned)((n_rows + 3) / 4);
+  const unsigned blocks = (unsigned)n_rows;
 #define XI_RN(TI, TO) \
   rows_rmsnorm_kernel<TI, TO><<<blocks, 256, 0, stream>>>((const TI*)x, x_stride, w, eps, (TO*)out, n_rows, n)
   if (in_dtype == kF32 && out_dtype == kF32) XI_RN(float, float);

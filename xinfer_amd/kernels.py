@@ -1082,12 +1082,19 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
     `split_keys` > 0 (steps in which every sequence brings one token, a tile a token): each workgroup walks one slice
     of that many keys of the up to `span` a token sees, and a second kernel puts the slices together.
     `rows_heads` H > 0 (one kv head, single tokens): q is [tokens * H, 1, d], a sequence's H rows are the query heads
-    of its one new token, all at its last position, `cu_q` counts rows, `sinks` is [H] and blocks may hold many rows."""
+    of its one new token, all at its last position, `cu_q` counts rows, `sinks` is [H] and blocks may hold many rows.
+    The V pool may then have G > 1 heads beside the one key head: rows h H / G .. (h + 1) H / G - 1 read value head h, and
+    no block of `tiles` may cross such a border."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out, slopes, sinks)
     T, nq, d = q.shape
     nkk, nkv, page, dv = int(k_cache.shape[1]), int(vt_cache.shape[1]), k_cache.shape[2], int(vt_cache.shape[3])
     if nkk <= 0 or nkv % nkk:
         raise KernelError(f"attention_biased: {nkv} kv heads on {nkk} key heads")
+    rows_kv = 1
+    if rows_heads and nkk == 1 and nkv > 1:         # heads as rows over one key head and several value heads
+        if int(rows_heads) % nkv:
+            raise KernelError(f"attention_biased: {rows_heads} heads as rows on {nkv} value heads")
+        rows_kv, nkv = nkv, 1
     _want(q, torch.bfloat16, "attention_biased: q")
     if sinks is not None:
         _want(sinks, torch.float32, "attention_biased: sinks")
@@ -1095,7 +1102,7 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
             raise KernelError(f"attention_biased: sinks {tuple(sinks.shape)} must be one a query head, [{int(rows_heads) or nq}]")
     if rows_heads and (nq != 1 or nkv != 1 or slopes is not None or T % int(rows_heads)):
         raise KernelError("attention_biased: rows that are a token's heads come with one head, no slopes and whole tokens")
-    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_biased", dv=dv, key_heads=nkk)
+    _check_cache(k_cache, vt_cache, nkv * rows_kv, d, torch.bfloat16, True, "attention_biased", dv=dv, key_heads=nkk)
     for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
         _want(t, torch.int32, f"attention_biased: {name}")
     B = ctx_lens.shape[0]
@@ -1126,7 +1133,7 @@ def attention_biased_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_l
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles), int(tiles.shape[0]),
         _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), ctypes.c_float(softcap), _p(slopes), _p(sinks), int(window),
         int(page), nq, nkv, d, dv, int(small), _p(part_o), _p(part_ml), int(split_keys), int(max_splits), int(T), int(rows_heads),
-        nkk, _stream()))
+        nkk, rows_kv, _stream()))
     return out
 
 
@@ -1236,6 +1243,31 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     if softcap > 0 or slopes is not None or sinks is not None or v_cache.shape[3] != d or nkk != nkv:
         dv = int(v_cache.shape[3])
         if q.dtype == torch.bfloat16 and v_grouped and BIASED_MFMA and attention_biased_supported(nq, nkv, d, dv, page):
+            if (ctx.max_q_len == 1 and nkk == 1 and nkv > 1 and nq // nkv >= HEAD_ROWS_FROM and slopes is None and sinks is None
+                    and q.is_contiguous()):
+                # single tokens whose heads all read the one key head and, group by group, a value head of their own:
+                # a group's heads are the rows of its blocks, so a tile of keys is read once a group and not once
+                # for every few heads
+                per = nq // nkv
+                key = ("attention_biased_group_rows", d, dv, nq, nkv)
+                cached = ctx.scratch.get(key)
+                if cached is None:
+                    small = 1 if attention_biased_block(d, dv, 1, 1) >= per else 0
+                    rows = attention_biased_block(d, dv, 1, small)
+                    nb = -(-per // rows)                    # blocks a group; made on the device: the step may be recorded
+                    blocks = nkv * nb
+                    firsts = (torch.arange(nkv, dtype=torch.int32, device=q.device).repeat_interleave(nb) * per
+                              + torch.arange(nb, dtype=torch.int32, device=q.device).repeat(nkv) * rows)
+                    seqs = torch.arange(ctx.num_seqs, dtype=torch.int32, device=q.device).repeat_interleave(blocks)
+                    first = firsts.repeat(ctx.num_seqs)
+                    cached = (torch.stack([seqs, first], dim=1).contiguous(), small, ctx.cu_q * nq, blocks)
+                    ctx.scratch[key] = cached
+                tiles, small, cu_rows, blocks = cached
+                span = min(int(ctx.max_ctx_len), int(window) + 63) if window > 0 else int(ctx.max_ctx_len)
+                split = biased_split_keys(ctx.num_seqs * blocks, span)
+                out = attention_biased_bf16(q.view(T * nq, 1, d), k_cache, v_cache, bt, tiles, cu_rows, ctx.ctx_lens, scale, window,
+                                            softcap=softcap, small=small, split_keys=split, span=span, rows_heads=nq)
+                return out.view(T, nq * dv)
             if ctx.max_q_len == 1 and nkv == 1 and nq >= HEAD_ROWS_FROM and slopes is None and q.is_contiguous():
                 # single tokens whose heads all read the one kv head: the heads are the rows of a block, so a tile
                 # of keys is read once for all of them (nothing of the step is read on the host)
