@@ -24,31 +24,11 @@
 
 namespace xi {
 
-constexpr int kRowThreads = 1024;   // a token's row is a few thousand channels: every thread a few, all loads in flight at once
+// threads a token: 1024 in steps of few tokens (a row is a few thousand channels: every thread a few, their loads in flight
+// at once), 256 where the tokens themselves fill the chip
 constexpr int kTapsUnrolled = 8;    // convolutions of up to this many taps ask for all their inputs before the first sum
 
-template <typename T>
-__device__ __forceinline__ void store_run8(T* dst, const float (&v)[8]) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) dst[i] = from_float<T>(v[i]);
-}
-template <>
-__device__ __forceinline__ void store_run8<bf16>(bf16* dst, const float (&v)[8]) {      // 16 bytes where the place allows it
-  if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
-    unsigned u[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const bf16 lo = __float2bfloat16(v[2 * i]), hi = __float2bfloat16(v[2 * i + 1]);
-      u[i] = (unsigned)*reinterpret_cast<const unsigned short*>(&lo) | ((unsigned)*reinterpret_cast<const unsigned short*>(&hi) << 16);
-    }
-    *reinterpret_cast<uint4*>(dst) = make_uint4(u[0], u[1], u[2], u[3]);
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) dst[i] = __float2bfloat16(v[i]);
-  }
-}
-
-template <typename T>
+template <typename T, int kRowThreads>
 __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
     const T* __restrict__ u, long long u_stride, const float* __restrict__ cw, int taps, const float* __restrict__ tails,
     long long tail_stride, const long long* __restrict__ state_slots, const int* __restrict__ tok_seq,
@@ -63,23 +43,33 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
   if (talk)
     for (int i = threadIdx.x; i < nq * nq; i += kRowThreads) talk_s[i] = talk[i];
   const T* ur = u + (size_t)t * u_stride;
-  if (taps > 1 && taps <= kTapsUnrolled) {
+  if (taps > 1 && taps <= kTapsUnrolled) {       // four channels a thread at a time, all their inputs asked for before the first sum
     const int b = tok_seq[t];
     const int t0 = cu_q[b];
     const float* tail = tails + (size_t)state_slots[b] * tail_stride;
-    for (int c = threadIdx.x; c < C; c += kRowThreads) {
-      float x[kTapsUnrolled], w[kTapsUnrolled];
+    constexpr int kAtOnce = 4;
+    for (int c0 = threadIdx.x; c0 < C; c0 += kAtOnce * kRowThreads) {
+      float x[kAtOnce][kTapsUnrolled], w[kAtOnce][kTapsUnrolled];
 #pragma unroll
-      for (int j = 0; j < kTapsUnrolled; ++j) {
-        const int s = t - (taps - 1) + j;
-        x[j] = j >= taps ? 0.f : s >= t0 ? to_float(u[(size_t)s * u_stride + c]) : tail[(size_t)(taps - 1 - (t0 - s)) * C + c];
-        w[j] = j < taps ? cw[(size_t)c * taps + j] : 0.f;
+      for (int a = 0; a < kAtOnce; ++a) {
+        const int c = c0 + a * kRowThreads;
+#pragma unroll
+        for (int j = 0; j < kTapsUnrolled; ++j) {
+          const int s = t - (taps - 1) + j;
+          const bool in = j < taps && c < C;
+          x[a][j] = !in ? 0.f : s >= t0 ? to_float(u[(size_t)s * u_stride + c]) : tail[(size_t)(taps - 1 - (t0 - s)) * C + c];
+          w[a][j] = in ? cw[(size_t)c * taps + j] : 0.f;
+        }
       }
-      float acc = 0.f;
 #pragma unroll
-      for (int j = 0; j < kTapsUnrolled; ++j)
-        if (j < taps) acc = fmaf(w[j], x[j], acc);
-      row[c] = acc;
+      for (int a = 0; a < kAtOnce; ++a) {
+        const int c = c0 + a * kRowThreads;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < kTapsUnrolled; ++j)
+          if (j < taps) acc = fmaf(w[a][j], x[a][j], acc);
+        if (c < C) row[c] = acc;
+      }
     }
   } else if (taps > 1) {
     const int b = tok_seq[t];
@@ -120,20 +110,31 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
     }
   }
   __syncthreads();
-  if (talk && d % 8 == 0) {                      // eight dims of one (head, kv head) a thread
-    const int g = nq / nkv;                      // query heads on a kv head
+  if (talk && d % 4 == 0 && nq % 4 == 0) {       // four heads by four dims of one kv head a thread: a small product a token,
+    const int g = nq / nkv;                      // its operands read from LDS once for sixteen sums
     T* qo = q_out + (size_t)t * nq * nkd;
-    for (int i = threadIdx.x; i < nq * nkd / 8; i += kRowThreads) {
-      const int h = (8 * i) / nkd, r = 8 * i - h * nkd;
+    const int per_row = nkd / 4;
+    for (int i = threadIdx.x; i < (nq / 4) * per_row; i += kRowThreads) {
+      const int hb = i / per_row, r = 4 * (i - hb * per_row);
       const int c = r / d, e = r - c * d;
-      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float acc[4][4] = {};
       for (int j = 0; j < g; ++j) {
-        const float w = talk_s[h * nq + c * g + j];
-        const float* src = row + (c * g + j) * d + e;
+        const float4 x = *reinterpret_cast<const float4*>(row + (c * g + j) * d + e);
 #pragma unroll
-        for (int x = 0; x < 8; ++x) acc[x] = fmaf(w, src[x], acc[x]);
+        for (int a = 0; a < 4; ++a) {
+          const float w = talk_s[(4 * hb + a) * nq + c * g + j];
+          acc[a][0] = fmaf(w, x.x, acc[a][0]);
+          acc[a][1] = fmaf(w, x.y, acc[a][1]);
+          acc[a][2] = fmaf(w, x.z, acc[a][2]);
+          acc[a][3] = fmaf(w, x.w, acc[a][3]);
+        }
       }
-      store_run8<T>(qo + 8 * i, acc);
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        T* dst = qo + (size_t)(4 * hb + a) * nkd + r;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) dst[x] = from_float<T>(acc[a][x]);
+      }
     }
   } else if (talk) {
     const int g = nq / nkv;
@@ -226,12 +227,17 @@ int xi_conv_qkv_rows(const void* u, long long u_stride, int dtype, const float* 
   if (n_tok == 0) return 0;
 #define XI_CR(TT)                                                                                                     \
   do {                                                                                                                \
-    auto kern = conv_qkv_rows_kernel<TT>;                                                                             \
+    if (n_tok <= 128) XI_CR_N(TT, 1024);                                                                              \
+    else XI_CR_N(TT, 256);                                                                                            \
+  } while (0)
+#define XI_CR_N(TT, NT)                                                                                               \
+  do {                                                                                                                \
+    auto kern = conv_qkv_rows_kernel<TT, NT>;                                                                         \
     if (lds > 48 * 1024) {                                                                                            \
       hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
       XI_CHECK(e_ == hipSuccess, "conv_qkv_rows: cannot get %zu bytes of LDS", lds);                                  \
     }                                                                                                                 \
-    kern<<<n_tok, kRowThreads, lds, stream>>>((const TT*)u, u_stride, cw, taps, tails, tail_stride, state_slots, tok_seq, \
+    kern<<<n_tok, NT, lds, stream>>>((const TT*)u, u_stride, cw, taps, tails, tail_stride, state_slots, tok_seq, \
                                               cu_q, qw, kw, eps, v_unit, talk, slots, (TT*)q_out, (TT*)k_cache,       \
                                               (TT*)v_cache, page_size, nq, nkv, d, dv, v_grouped);                    \
   } while (0)
@@ -239,6 +245,7 @@ int xi_conv_qkv_rows(const void* u, long long u_stride, int dtype, const float* 
   else if (dtype == kBF16) XI_CR(bf16);
   else XI_CHECK(false, "conv_qkv_rows: unknown dtype %d", dtype);
 #undef XI_CR
+#undef XI_CR_N
   XI_LAUNCH_CHECK("conv_qkv_rows");
   return 0;
 }

@@ -17,7 +17,7 @@
 
 namespace xi {
 
-constexpr int kGateBlock = 256;
+constexpr int kGateBlock = 1024;     // tokens a round: the chain of a round runs while nothing else does, so rounds are few
 
 __device__ __forceinline__ float log_sigmoid(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
@@ -43,9 +43,23 @@ __global__ __launch_bounds__(kGateBlock) void mlstm_gates_kernel(const float* __
       lk[threadIdx.x] = log_sigmoid(cap * tanhf((zr[H + h] + bf) * inv_cap));
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0) {              // eight tokens' gates asked for at once: the chain waits for no read
       float m = ms[0];
-      for (int i = 0; i < n; ++i) {
+      int i = 0;
+      for (; i + 8 <= n; i += 8) {
+        float keep8[8], in8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          keep8[e] = lk[i + e];
+          in8[e] = li[i + e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          m = fmaxf(keep8[e] + m, in8[e]);
+          ms[i + 1 + e] = m;
+        }
+      }
+      for (; i < n; ++i) {
         m = fmaxf(lk[i] + m, li[i]);
         ms[i + 1] = m;
       }
