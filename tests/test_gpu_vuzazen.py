@@ -244,7 +244,7 @@ def _folded_queries(q, talk, G):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,d,dv,taps,page,norms,talks", [
     (6, 2, 16, 24, 3, 16, True, True), (5, 5, 20, 20, 2, 8, True, True), (3, 1, 12, 20, 5, 8, True, True),
-    (4, 2, 8, 16, 1, 16, True, True), (4, 2, 128, 64, 3, 64, True, True), (6, 3, 8, 16, 4, 8, False, False), (2, 2, 16, 8, 3, 8, True, False)])
+    (4, 2, 8, 16, 1, 16, True, True), (4, 2, 8, 24, 0, 16, True, True), (4, 2, 128, 64, 3, 64, True, True), (6, 3, 8, 16, 4, 8, False, False), (2, 2, 16, 8, 3, 8, True, False)])
 def test_rows_after_the_convolution_the_norms_and_the_heads_mix(H, G, d, dv, taps, page, norms, talks, dtype):
     """A request in portions (some shorter than the taps), beside another request whose tail must not be touched: q (or
     q' with mixed heads) and what the cache holds against the plain convolution, norms and unit values."""
@@ -259,7 +259,7 @@ def test_rows_after_the_convolution_the_norms_and_the_heads_mix(H, G, d, dv, tap
     qw, kw = (1 + 0.3 * torch.randn(H * d, generator=g), 1 + 0.3 * torch.randn(G * d, generator=g)) if norms else (None, None)
     talk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).to(torch.bfloat16).float() if talks else None
     u = packed[:, :C].double()
-    y = plain.short_conv(u, cw.double()) if taps > 1 else u
+    y = plain.short_conv(u, cw.double()) if taps >= 1 else u          # one tap: a factor a channel; none: no convolution
     q, k, v = y[:, :H * d], y[:, H * d:H * d + G * d], y[:, H * d + G * d:].view(L, G, dv)
     if norms:
         q, k = plain.rms_norm(q, eps, qw.double()), plain.rms_norm(k, eps, kw.double())
@@ -278,7 +278,7 @@ def test_rows_after_the_convolution_the_norms_and_the_heads_mix(H, G, d, dv, tap
         sl = slots[at:at + n].clone()
         if at <= 5 < at + n:
             sl[5 - at] = -1                                                   # a token that stores nothing
-        qo = kernels.conv_qkv_rows(rows, cw.to(DEV) if taps > 1 else None, tails, _i64([1]), _i32([0] * n), _i32([0, n]),
+        qo = kernels.conv_qkv_rows(rows, cw.to(DEV) if taps >= 1 else None, tails, _i64([1]), _i32([0] * n), _i32([0, n]),
                                    None if qw is None else qw.to(DEV), None if kw is None else kw.to(DEV), eps, sl.to(DEV), k_pool, v_pool,
                                    H, G, d, dv, v_grouped=grouped, value_unit_norm=True, talk=None if talk is None else talk.to(DEV))
         if taps > 1:

@@ -12,7 +12,7 @@ M: memories alone (no layer keeps pages): requests have states and lengths, and 
 R: real-looking head sizes (64 and 128, a latent of 112 + 16, memories of 64 by 96 and 128 by 64) with pages of 64, for the
    matrix-core kernels; mixed heads over two kv heads of 128 (one key head of 256).
 S: the matrix-core kernels' sizes again: three kv heads of 32 with values of 128 and four query heads each (single
-   tokens then take a group's heads as the rows of a block), four kv heads of 64 that are all the heads, 4 taps, 3 of 8
+   tokens then take a group's heads as the rows of a block), four kv heads of 64 that are all the heads, 4 taps and one tap, 3 of 8
    experts.
 
 Random routers would leave some token's choice of experts to a difference that bfloat16 does not keep: `make_model`
@@ -93,7 +93,7 @@ MODELS = {
         seed=35, linear_std=0.04, norm_std=0.1, page_size=64),
     "S": dict(config=_config(300, 320, 1e-5, 10.0, (601, 17, 129), [
         _att(12, 3, 32, 128, 0.18, 4, _moe(64, 8, 3)),
-        _att(4, 4, 64, 64, 0.12, 2, _dense(320)),
+        _att(4, 4, 64, 64, 0.12, 1, _dense(320)),
         _lat(5, 48, 32, 64, 80, 56, 0.14, 500000.0, None)]),
         seed=36, linear_std=0.05, norm_std=0.1, page_size=64),
 }

@@ -5,7 +5,7 @@
 //                 [C, taps], no bias, no activation); inputs from before the step's portion come from the request's
 //                 tail (the last taps - 1 projected rows of earlier steps, float32 [slots, taps - 1, C], oldest first;
 //                 zeros for a request's first tokens).  `conv_tail_kernel` (ssm.hip) moves the tail on afterwards.
-//                 taps <= 1: none.
+//                 One tap is a factor a channel and needs no tail; no weights: no convolution.
 //   norms         RMS norm over the WHOLE q part and the whole k part (one mean over all heads, weights qw [nq d] and
 //                 kw [nkv d]; null: none); with `v_unit` every value head divided by its own root mean square over dv;
 //                 eps inside the roots.
@@ -43,10 +43,10 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
   if (talk)
     for (int i = threadIdx.x; i < nq * nq; i += kRowThreads) talk_s[i] = talk[i];
   const T* ur = u + (size_t)t * u_stride;
-  if (taps > 1 && taps <= kTapsUnrolled) {       // four channels a thread at a time, all their inputs asked for before the first sum
-    const int b = tok_seq[t];
-    const int t0 = cu_q[b];
-    const float* tail = tails + (size_t)state_slots[b] * tail_stride;
+  if (cw && taps <= kTapsUnrolled) {             // four channels a thread at a time, all their inputs asked for before the first sum
+    const int b = taps > 1 ? tok_seq[t] : 0;
+    const int t0 = taps > 1 ? cu_q[b] : 0;
+    const float* tail = taps > 1 ? tails + (size_t)state_slots[b] * tail_stride : nullptr;
     constexpr int kAtOnce = 4;
     for (int c0 = threadIdx.x; c0 < C; c0 += kAtOnce * kRowThreads) {
       float x[kAtOnce][kTapsUnrolled], w[kAtOnce][kTapsUnrolled];
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
         if (c < C) row[c] = acc;
       }
     }
-  } else if (taps > 1) {
+  } else if (cw) {
     const int b = tok_seq[t];
     const int t0 = cu_q[b];
     const float* tail = tails + (size_t)state_slots[b] * tail_stride;
@@ -204,8 +204,8 @@ using namespace xi;
 
 extern "C" {
 
-// u: rows of u_stride elements in `dtype`, the first C = nq d + nkv d + nkv dv are q, k, v; cw float32 [C, taps] (taps
-// <= 1: unused); tails float32, slot s at tails + s * tail_stride, [taps - 1, C]; state_slots int64 [B]; tok_seq int32
+// u: rows of u_stride elements in `dtype`, the first C = nq d + nkv d + nkv dv are q, k, v; cw float32 [C, taps] (null:
+// no convolution); tails float32, slot s at tails + s * tail_stride, [taps - 1, C]; state_slots int64 [B]; tok_seq int32
 // [T]; cu_q int32 [B + 1]; qw, kw float32 or both null; talk float32 [nq, nq] or null; slots int64 [T]; q_out [T, nq,
 // nkv d] with talk, else [T, nq, d]; pools as the head of the file says.
 int xi_conv_qkv_rows(const void* u, long long u_stride, int dtype, const float* cw, int taps, const float* tails,
@@ -218,8 +218,9 @@ int xi_conv_qkv_rows(const void* u, long long u_stride, int dtype, const float* 
   const long long C = (long long)nq * d + (long long)nkv * d + (long long)nkv * dv;
   XI_CHECK(u_stride >= C, "conv_qkv_rows: rows of %lld elements do not hold %lld channels", u_stride, C);
   XI_CHECK((qw == nullptr) == (kw == nullptr), "conv_qkv_rows: q and k norm weights must both be given or both absent");
-  XI_CHECK(taps <= 1 || (cw && tails && state_slots && tok_seq && cu_q && tail_stride >= (taps - 1) * C),
-           "conv_qkv_rows: a convolution of %d taps needs its weights and the requests' tails", taps);
+  XI_CHECK(cw == nullptr || taps >= 1, "conv_qkv_rows: a convolution of %d taps", taps);
+  XI_CHECK(cw == nullptr || taps == 1 || (tails && state_slots && tok_seq && cu_q && tail_stride >= (taps - 1) * C),
+           "conv_qkv_rows: a convolution of %d taps needs the requests' tails", taps);
   XI_CHECK(!v_grouped || page_size % 8 == 0, "conv_qkv_rows: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d",
            page_size);
   const size_t lds = ((size_t)C + (talk ? (size_t)nq * nq : 0)) * sizeof(float);

@@ -2025,8 +2025,8 @@ def conv_qkv_rows(qkv: torch.Tensor, conv_weight: Optional[torch.Tensor], tails:
                   num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, v_grouped: bool = False,
                   value_unit_norm: bool = False, talk: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The first nq d + nkv d + nkv dv columns of a packed projection made ready for attention: a causal convolution per
-    channel over the last `taps` tokens (`conv_weight` float32 [C, taps]; None: none; inputs from before the step come
-    from `tails` float32 [slots, taps - 1, C] at `state_slots`, which `conv_tail` moves on afterwards), RMSNorm over the
+    channel over the last `taps` tokens (`conv_weight` float32 [C, taps]; None: none; one tap: a factor a channel; inputs
+    from before the step come from `tails` float32 [slots, taps - 1, C] at `state_slots`, which `conv_tail` moves on afterwards), RMSNorm over the
     whole q part and the whole k part (weights float32; None: none), every value head divided by its root mean square
     (`value_unit_norm`), k and v into the paged cache at `slots`.  With `talk` float32 [nq, nq] (head h's score is
     sum_g talk[h, g] (q_g . k)) the sum is taken on the query's side: the result is q' [T, nq, nkv d] and the K pool

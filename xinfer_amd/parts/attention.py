@@ -26,9 +26,9 @@ rounding); with the options of the paragraph above, or with `general=True`, a ke
 it in the order given (`kernels.head_rows`: rotation of either pairing, then the unit norm, then the cache write).
 
 A third group of options, each a parameter of the spec, goes through `_forward_rows` (no rotation, `qk_norm` "row" or
-none): `conv` n > 1: q, k and v pass a causal convolution per channel over the last n tokens right after the
+none): `conv` n: q, k and v pass a causal convolution per channel over the last n tokens right after the
 projection (tensors `q_conv`, `k_conv`, `v_conv` [channels, n], no bias; the last n - 1 projected rows of a request are
-state of the layer, "conv_tail"); `value_norm="head_unit"`: every value head is divided by its root mean square and
+state of the layer, "conv_tail"; one tap is a factor a channel and keeps nothing); `value_norm="head_unit"`: every value head is divided by its root mean square and
 cached so; `talking_heads`: head h's score of a key is sum_g talk[h, g] * (head g's score) before the softmax (tensor
 `talk` [heads, heads]); `head_gate`: head h's result times sigmoid(w_h . x), one number a head (tensor `head_gate`
 [heads, hidden], packed with q, k and v).  The heads' sum moves to the query's side, q'_h = [sum_{g on kv head c}
@@ -96,7 +96,7 @@ class PagedAttention(Mixer):
         self.talking = bool(spec.get("talking_heads", False))
         self.head_gate = bool(spec.get("head_gate", False))
         # a convolution, normed values, mixed heads or a gate a head: one kernel makes a token's row ready
-        self.rows_form = self.taps > 1 or self.value_unit or self.talking or self.head_gate
+        self.rows_form = self.taps >= 1 or self.value_unit or self.talking or self.head_gate
         if self.rows_form:
             self.general = True
             if (self.by_head or spec.get("position") is not None or self.softcap > 0 or self.slope_values is not None
@@ -157,7 +157,7 @@ class PagedAttention(Mixer):
         if vm and not vm.get("source", False):
             out.append(TensorDecl(n["value_mix"], (), "mix"))
         taps = int(spec.get("conv") or 0)
-        if taps > 1:
+        if taps >= 1:
             out += [TensorDecl(n["q_conv"], (nq * d, taps), "normal(0,0.5)"), TensorDecl(n["k_conv"], (nkv * d, taps), "normal(0,0.5)"),
                     TensorDecl(n["v_conv"], (nkv * dv, taps), "normal(0,0.5)")]
         if spec.get("talking_heads", False):
@@ -172,7 +172,7 @@ class PagedAttention(Mixer):
             return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
         names = self._names(self.spec, prefix)
         parts = [lin(names[n]) for n in (("q", "k", "v", "head_gate") if self.head_gate else ("q", "k", "v"))]
-        if self.taps > 1:
+        if self.taps >= 1:
             self.conv_w = torch.cat([store.get(names[n], torch.float32, device) for n in ("q_conv", "k_conv", "v_conv")]).contiguous()
         if self.talking:
             self.talk = store.get(names["talk"], torch.float32, device).contiguous()
