@@ -415,10 +415,13 @@ __global__ __launch_bounds__(64) void attn_biased_combine_kernel(const float* __
     __syncthreads();
     for (int i = lane; i < dv; i += 64) {
       float o = 0.f;
-#pragma unroll 4
+      // every slice's sum is asked for, eight at a time (a slice without keys left its place unwritten: what is read
+      // there is not used)
+#pragma unroll 8
       for (int s2 = 0; s2 < max_splits; ++s2) {
         const float fs = f_s[s2];
-        if (fs > 0.f) o += part_o[(base + s2) * dv + i] * fs;
+        const float v = part_o[(base + s2) * dv + i];
+        o += fs > 0.f ? v * fs : 0.f;
       }
       out[((size_t)t * nq + head) * dv + i] = __float2bfloat16(o * inv);
     }
