@@ -28,6 +28,30 @@ namespace xi {
 // at once), 256 where the tokens themselves fill the chip
 constexpr int kTapsUnrolled = 8;    // convolutions of up to this many taps ask for all their inputs before the first sum
 
+// four values that follow each other, in one store where the type and the place allow it
+__device__ __forceinline__ void store_run4(float* dst, const float (&v)[4]) {
+  if ((reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = v[i];
+  }
+}
+__device__ __forceinline__ void store_run4(bf16* dst, const float (&v)[4]) {
+  if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+    unsigned u[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const bf16 lo = __float2bfloat16(v[2 * i]), hi = __float2bfloat16(v[2 * i + 1]);
+      u[i] = (unsigned)*reinterpret_cast<const unsigned short*>(&lo) | ((unsigned)*reinterpret_cast<const unsigned short*>(&hi) << 16);
+    }
+    *reinterpret_cast<uint2*>(dst) = make_uint2(u[0], u[1]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[i] = __float2bfloat16(v[i]);
+  }
+}
+
 template <typename T, int kRowThreads>
 __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
     const T* __restrict__ u, long long u_stride, const float* __restrict__ cw, int taps, const float* __restrict__ tails,
@@ -130,11 +154,7 @@ __global__ __launch_bounds__(kRowThreads) void conv_qkv_rows_kernel(
         }
       }
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        T* dst = qo + (size_t)(4 * hb + a) * nkd + r;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) dst[x] = from_float<T>(acc[a][x]);
-      }
+      for (int a = 0; a < 4; ++a) store_run4(qo + (size_t)(4 * hb + a) * nkd + r, acc[a]);
     }
   } else if (talk) {
     const int g = nq / nkv;
