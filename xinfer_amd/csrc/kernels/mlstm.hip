@@ -7,7 +7,8 @@
 //     m' = max(log_keep + m, log_in)             (m: a running maximum, state of the request, 0 when it starts)
 //     keep = exp(log_keep + m - m')   take = exp(log_in - m')   floor = exp(-m')
 // and writes (keep, take) [T, H, 2] and floor [T, H].  The chain over m is two operations a token and is walked by
-// one thread; logits before and exponentials after are made by the whole workgroup, a block of tokens at a time.
+// one wave, 64 tokens' gates in its lanes' registers at a time; logits before and exponentials after are made by the
+// whole workgroup, a block of tokens at a time.
 // Everything float32: what a token gets does not depend on how the prompt was cut, bit for bit.
 //
 // `mlstm_finish_kernel`: o [T, H, dv + 1] float32 (the state's results; the last column is n . q):
@@ -43,25 +44,19 @@ __global__ __launch_bounds__(kGateBlock) void mlstm_gates_kernel(const float* __
       lk[threadIdx.x] = log_sigmoid(cap * tanhf((zr[H + h] + bf) * inv_cap));
     }
     __syncthreads();
-    if (threadIdx.x == 0) {              // eight tokens' gates asked for at once: the chain waits for no read
-      float m = ms[0];
-      int i = 0;
-      for (; i + 8 <= n; i += 8) {
-        float keep8[8], in8[8];
+    if (threadIdx.x < kWave) {           // the first wave walks the chain: lane l holds token l's gates of a run of 64, every
+      float m = ms[0];                   // lane follows the whole chain (the gates reach it from the lanes' registers, not
+      for (int first = 0; first < n; first += kWave) {     // from memory) and keeps its own token's value
+        const int i = first + (int)threadIdx.x;
+        const int keep_bits = __float_as_int(i < n ? lk[i] : 0.f);            // past the end: m stays what it is
+        const int in_bits = __float_as_int(i < n ? li[i] : -INFINITY);
+        float mine = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          keep8[e] = lk[i + e];
-          in8[e] = li[i + e];
+        for (int e = 0; e < kWave; ++e) {
+          m = fmaxf(__int_as_float(__builtin_amdgcn_readlane(keep_bits, e)) + m, __int_as_float(__builtin_amdgcn_readlane(in_bits, e)));
+          if ((int)threadIdx.x == e) mine = m;
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          m = fmaxf(keep8[e] + m, in8[e]);
-          ms[i + 1 + e] = m;
-        }
-      }
-      for (; i < n; ++i) {
-        m = fmaxf(lk[i] + m, li[i]);
-        ms[i + 1] = m;
+        if (i < n) ms[i + 1] = mine;
       }
     }
     __syncthreads();
