@@ -20,7 +20,7 @@ def rms_norm(x, eps, w=None):
 
 
 def layer_norm_weight(w):
-    """The layers' norms store their weight around zero: the factor is 1 + w."""
+    """A norm's tensor holds its factor's distance from one: the factor is 1 + w."""
     return 1.0 + w
 
 

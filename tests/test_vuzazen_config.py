@@ -46,14 +46,14 @@ def test_what_the_layers_keep_and_what_their_tensors_are_called():
     assert model.blocks[1].mixer.rows_form and model.blocks[3].mixer.taps == 0 and model.blocks[3].mixer.state_need() is None
     assert model.blocks[2].mixer.head_gate and model.blocks[2].mixer.q_rank == 24 and not model.blocks[2].mixer.has_sinks
     assert model.blocks[0].ffn.sigmoid_scores and model.blocks[0].ffn.weigh_input
-    # every norm of the family has its weight stored around zero
+    # every norm of the family multiplies by one plus its tensor
     assert model.blocks[0].norm1.weight_offset == 1.0 and model.final_norm.weight_offset == 1.0
     fam, cfg = config_from_dict(MODELS["M"]["config"])
     model = CausalLM(fam.spec(cfg), torch.bfloat16)
     assert not model.kv_needs and sorted(model.state_needs) == [EMBEDDING_CACHE, 0, 1]
 
 
-def test_a_norm_weight_stored_around_zero():
+def test_a_norm_that_multiplies_by_one_plus_its_tensor():
     from xinfer_amd.config.spec import PartSpec
     from xinfer_amd.parts import norm_class
     from xinfer_amd.weights.store import RandomStore

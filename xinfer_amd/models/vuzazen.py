@@ -7,8 +7,8 @@ there:
   embedding   x = embed[token] * embedding.scale + bigram[row], row = (previous token * mul_prev + token * mul_cur) mod
               buckets, and row `buckets` (the table's last) for a sequence's first token
   layer       pre-norm: x <- x + mixer(norm1(x)), then x <- x + ff(norm2(x)); `mlp: null` leaves the second out;
-              every norm (the model's last one too) is x * rsqrt(mean(x^2) + eps) * (1 + w): the stored weight lies
-              around zero
+              every norm (the model's last one too) is x * rsqrt(mean(x^2) + eps) * (1 + w): the tensor holds the
+              factor's distance from one
   type "mlstm"             a matrix memory per head (`parts/mlstm.py`): exponential input gate, sigmoid forget gate,
               both logits capped by gate_cap * tanh(. / gate_cap), a running maximum that keeps the exponentials in
               range; q scaled by dim^-1/2; the heads' results divided by their root mean square, times a weight, times

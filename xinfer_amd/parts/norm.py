@@ -4,7 +4,7 @@ out = s * rsqrt(mean(s^2) + eps) * w with s = resid (+ add), everything in float
 one rounding to the output type (reference: NormX::forward and forward_add,
 /root/reference/src/models/layers/others.rs:22-62; weight kept in float32,
 /root/reference/src/models/qwen3.rs:83).  With `weight_offset` c the stored tensor lies around -c + 1
-and the factor is c + w (c = 1: a weight stored around zero); the sum is made once, in float32, when the
+and the factor is c + w (c = 1: the tensor is the factor's distance from one); the sum is made once, in float32, when the
 tensor is loaded.
 """
 from __future__ import annotations
