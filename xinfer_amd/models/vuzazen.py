@@ -124,7 +124,7 @@ class ConvAttentionMixer:
     dim: int
     vdim: int
     scale: float
-    conv: int                          # taps of the convolution over time; 0 or 1: none
+    conv: int                          # taps of the convolution over time; 0: none (one tap: a factor a channel)
 
     @classmethod
     def from_dict(cls, raw: Any, where: str) -> "ConvAttentionMixer":
